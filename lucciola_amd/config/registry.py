@@ -74,10 +74,11 @@ BLOCKS: Registry[type] = Registry("block arrangement")
 EMBEDDINGS: Registry[type] = Registry("embedding")
 HEADS: Registry[type] = Registry("output head")
 STREAM_STEPS: Registry[type] = Registry("stream step")
+INPUT_SHIFTS: Registry[type] = Registry("input shift")
 
 # the families a block's slots may name
 FAMILIES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
-            "position": POSITION_ENCODINGS}
+            "position": POSITION_ENCODINGS, "input_shift": INPUT_SHIFTS}
 
 
 def architecture_for(config_dict: Dict[str, Any]) -> Architecture:

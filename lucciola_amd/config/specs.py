@@ -42,6 +42,18 @@ def mixer_only_layer(mixer: PartSpec, mixer_norm: PartSpec, names: Dict[str, str
     return LayerSpec("prenorm_mixer", {"mixer": mixer, "mixer_norm": mixer_norm}, names)
 
 
+def shifted_layer(mixer: PartSpec, feed_forward: Optional[PartSpec], mixer_norm: PartSpec,
+                  feed_forward_norm: Optional[PartSpec], mixer_shift: PartSpec, names: Dict[str, str]) -> LayerSpec:
+    """A pre-norm layer whose mixer reads its normed input through an input shift (``prenorm_shift_residual``,
+    or ``prenorm_shift_mixer`` without a feed-forward)."""
+    if feed_forward is None:
+        return LayerSpec("prenorm_shift_mixer", {"mixer": mixer, "mixer_norm": mixer_norm, "mixer_shift": mixer_shift},
+                         names)
+    return LayerSpec("prenorm_shift_residual",
+                     {"mixer": mixer, "feed_forward": feed_forward, "mixer_norm": mixer_norm,
+                      "feed_forward_norm": feed_forward_norm, "mixer_shift": mixer_shift}, names)
+
+
 def prenorm_layer(mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
                   feed_forward_norm: PartSpec, names: Dict[str, str]) -> LayerSpec:
     """A layer in the pre-norm residual arrangement (``prenorm_residual``)."""
@@ -84,6 +96,7 @@ class ModelSpec:
     embedding: Optional[PartSpec] = None
     head: Optional[PartSpec] = None
     head_names: Optional[Dict[str, str]] = None   # a head with tensors beyond "weight" names them here
+    embedding_names: Optional[Dict[str, str]] = None   # likewise an embedding with tensors beyond its table
 
     def validate(self) -> None:
         for i, entry in enumerate(self.run_order):

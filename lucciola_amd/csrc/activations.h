@@ -6,7 +6,10 @@
 
 namespace lc {
 
-enum : int { ACT_NONE = 0, ACT_GELU_TANH = 1, ACT_RELU_SQUARED = 2, ACT_SIGMOID_GATE = 3 };
+// ACT_SIGMOID_GATE: times sigmoid of the gate's entry at the output's place; ACT_SIGMOID_GROUP_GATE: times
+// sigmoid of ONE gate entry per row and group (a number per token and head)
+enum : int { ACT_NONE = 0, ACT_GELU_TANH = 1, ACT_RELU_SQUARED = 2, ACT_SIGMOID_GATE = 3, ACT_SIGMOID_GROUP_GATE = 4,
+             ACT_XIELU = 5 };
 
 __device__ __forceinline__ float activate(float z, int kind) {
     if (kind == ACT_GELU_TANH) {
@@ -21,5 +24,12 @@ __device__ __forceinline__ float activate(float z, int kind) {
 }
 
 __device__ __forceinline__ float sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
+
+// xIELU with its two numbers already through softplus: z > 0: a z^2 + z/2;  z <= 0: b (e^z - 1 - z) + z/2
+// (a = softplus(p), b = 1/2 + softplus(q)).
+__device__ __forceinline__ float xielu(float z, float a, float b) {
+    if (z > 0.f) return fmaf(a * z, z, 0.5f * z);
+    return fmaf(b, expm1f(z) - z, 0.5f * z);
+}
 
 }  // namespace lc

@@ -202,12 +202,13 @@ __global__ __launch_bounds__(THREADS) void rmsnorm_vec_kernel(
     }
 }
 
-// RMSNorm of rows held in the activation type (no residual stream involved).
+// RMSNorm of rows held in the activation type (no residual stream involved); a row of x begins every
+// `ld` entries (the first n columns of a wider tensor), the rows of out lie back to back.
 template <typename T>
-__global__ void rmsnorm_act_kernel(const T* __restrict__ x, const float* __restrict__ w,
+__global__ void rmsnorm_act_kernel(const T* __restrict__ x, long long ld, const float* __restrict__ w,
                                    float eps, T* __restrict__ out, int n) {
     __shared__ float scratch[16];
-    const T* xr = x + (size_t)blockIdx.x * n;
+    const T* xr = x + (size_t)blockIdx.x * ld;
     float ss = 0.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float v = to_f32(xr[i]);
@@ -465,16 +466,16 @@ LC_API int lc_rmsnorm(float* h, const void* delta, const int* rows, const float*
     return 0;
 }
 
-LC_API int lc_rmsnorm_act(const void* x, const float* w, float eps, void* out, int dt, int R,
+LC_API int lc_rmsnorm_act(const void* x, long long ld, const float* w, float eps, void* out, int dt, int R,
                           int n, hipStream_t stream) {
-    LC_CHECK(R >= 0 && n > 0, "rmsnorm_act: bad sizes R=%d n=%d", R, n);
+    LC_CHECK(R >= 0 && n > 0 && ld >= n, "rmsnorm_act: bad sizes R=%d n=%d", R, n);
     if (R == 0) return 0;
     LC_CHECK(x && w && out, "rmsnorm_act: null pointer");
     const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
     if (dt == DT_F32)
-        rmsnorm_act_kernel<float><<<R, threads, 0, stream>>>((const float*)x, w, eps, (float*)out, n);
+        rmsnorm_act_kernel<float><<<R, threads, 0, stream>>>((const float*)x, ld, w, eps, (float*)out, n);
     else if (dt == DT_BF16)
-        rmsnorm_act_kernel<bf16><<<R, threads, 0, stream>>>((const bf16*)x, w, eps, (bf16*)out, n);
+        rmsnorm_act_kernel<bf16><<<R, threads, 0, stream>>>((const bf16*)x, ld, w, eps, (bf16*)out, n);
     else
         LC_CHECK(false, "rmsnorm_act: unknown dtype %d", dt);
     LC_LAUNCH_CHECK("rmsnorm_act");

@@ -183,6 +183,7 @@ __global__ __launch_bounds__(256, 2) void gemm_grouped_kernel(GroupedArgs a) {
                 if (m < r_end && n < N) {
                     float v = total[i][j][r];
                     if (a.epilogue == ACT_SIGMOID_GATE) v *= sigmoid(to_f32(gate[(size_t)m * a.ldg + n]));
+                    else if (a.epilogue == ACT_SIGMOID_GROUP_GATE) v *= sigmoid(to_f32(gate[(size_t)m * a.ldg]));
                     else v = activate(v, a.epilogue);
                     out[(size_t)m * a.ldo + n] = from_f32<TO>(v);
                 }
@@ -302,6 +303,7 @@ __global__ __launch_bounds__(256, 2) void gemm_grouped_bf16_kernel(GroupedArgs a
                 if (m < r_end && n < N) {
                     float v = acc[i][j][r];
                     if (a.epilogue == ACT_SIGMOID_GATE) v *= sigmoid(to_f32(gate[(size_t)m * a.ldg + n]));
+                    else if (a.epilogue == ACT_SIGMOID_GROUP_GATE) v *= sigmoid(to_f32(gate[(size_t)m * a.ldg]));
                     else v = activate(v, a.epilogue);
                     out[(size_t)m * a.ldo + n] = from_f32<TO>(v);
                 }
@@ -370,8 +372,8 @@ LC_API int lc_gemm_grouped(const void* x, int x_dt, long long ldx, long long x_g
     LC_CHECK((row_start == nullptr) == (tile_start == nullptr), "grouped product: the lists come together");
     LC_CHECK(row_start || gather == nullptr, "grouped product: a gather list needs the rows' lists");
     LC_CHECK(!row_start || max_tiles > 0, "grouped product: no room for tiles");
-    LC_CHECK(epilogue >= ACT_NONE && epilogue <= ACT_SIGMOID_GATE, "grouped product: unknown epilogue %d", epilogue);
-    LC_CHECK(epilogue != ACT_SIGMOID_GATE || gate, "grouped product: no gates");
+    LC_CHECK(epilogue >= ACT_NONE && epilogue <= ACT_SIGMOID_GROUP_GATE, "grouped product: unknown epilogue %d", epilogue);
+    LC_CHECK((epilogue != ACT_SIGMOID_GATE && epilogue != ACT_SIGMOID_GROUP_GATE) || gate, "grouped product: no gates");
     LC_CHECK(tile_rows == 16 || tile_rows == 64 || tile_rows == 128, "grouped product: tiles of %d rows", tile_rows);
     LC_CHECK(G <= 65535 && (row_start ? max_tiles : (M + 15) / 16) <= 65535, "grouped product: too many tiles");
     GroupedArgs a{x, ldx, x_group, w, out, ldo, out_group, M, N, K, G, gather, row_start, tile_start,

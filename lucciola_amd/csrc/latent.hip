@@ -5,6 +5,8 @@
 // entries; q_r the rotated part, rot entries), so that for every head
 //   s_j = ([q_c | q_r] . [c_j | k_r,j]) * scale        over the keys j <= p, and j > p - window
 //   P = softmax(s),   o = sum_j P_j c_j                (R entries; W_uv is applied afterwards)
+// With a sink per head the softmax's denominator holds one more term, exp(sink): a key that has the
+// score `sink` (not scaled) whatever the query, and no value.
 // All heads of a token read the same rows.  Arithmetic is float32 throughout (scores, maximum,
 // exponentials, sums, P.c); only loads and stores have the tensors' type.
 //
@@ -22,20 +24,22 @@ constexpr int LA_KEYS = 64;       // keys of a chunk
 constexpr int LA_DIMS = 8;        // output entries a thread sums: R <= LA_THREADS * LA_DIMS
 
 // ------------------------------------------------------------------------------ prologue
-// One workgroup per token.  From the row [q heads | c' | k_r | ...] of the fused projection:
+// One workgroup per token.  From the token's rows of two tensors, [q heads ...] and [c' | k_r | ...] (the
+// same fused projection at two columns, or the queries from a product of their own):
 //   c = c' / sqrt(mean(c'^2) + eps) * w  and  rot(k_r) go to the token's cache row (slot >= 0);
 //   rot(q_r) of every head goes to qa[t][h][R ...].
 // Rotation of the first `rd` entries of a part: interleaved pairs (2i, 2i + 1) or halves
 // (i, i + rd/2), by the angle whose cosine and sine are table[p][i] and table[p][rd/2 + i].
 template <typename T>
 __global__ __launch_bounds__(LA_THREADS) void latent_prepare_kernel(
-    const T* __restrict__ proj, long long ld, int H, int dim, int rot, int R, const float* __restrict__ w,
+    const T* __restrict__ q, long long ldq, const T* __restrict__ kv, long long ld, int H, int dim, int rot, int R,
+    const float* __restrict__ w,
     float eps, const int* __restrict__ positions, const float* __restrict__ table, int rd, int interleaved,
     T* __restrict__ cache, const int* __restrict__ slots, T* __restrict__ qa) {
     __shared__ float scratch[16];
     const int t = blockIdx.x, tid = threadIdx.x;
-    const T* row = proj + (size_t)t * ld;
-    const T* down = row + (size_t)H * (dim + rot);
+    const T* row = q + (size_t)t * ldq;
+    const T* down = kv + (size_t)t * ld;
     const int Dk = R + rot;
     const long long slot = slots ? slots[t] : -1;
     T* mine = slot >= 0 ? cache + slot * Dk : nullptr;
@@ -77,7 +81,7 @@ template <typename T, bool VEC>
 __global__ __launch_bounds__(LA_THREADS) void latent_attention_kernel(
     const T* __restrict__ qa, int H, int R, int rot, const T* __restrict__ cache,
     const int* __restrict__ tok_req, const int* __restrict__ positions, const int* __restrict__ block_table,
-    int max_blocks, int page_size, float scale, int window, T* __restrict__ out) {
+    int max_blocks, int page_size, float scale, int window, const float* __restrict__ sink, T* __restrict__ out) {
     extern __shared__ float smem[];
     const int Dk = R + rot, Dp = (Dk + 3) & ~3;
     float* qs = smem;                                   // [LA_HEADS][Dp]
@@ -96,6 +100,10 @@ __global__ __launch_bounds__(LA_THREADS) void latent_attention_kernel(
         qs[i] = (hh < heads && e < Dk) ? to_f32(qa[((size_t)t * H + h0 + hh) * Dk + e]) * scale : 0.f;
     }
     float m_run = -INFINITY, l_run = 0.f;               // of head `wave`, the same in all its lanes
+    if (sink && wave < heads) {                         // the sink: seen before the first key, weight exp(0)
+        m_run = sink[h0 + wave];
+        l_run = 1.f;
+    }
     float acc[LA_HEADS][LA_DIMS];
 #pragma unroll
     for (int hh = 0; hh < LA_HEADS; ++hh)
@@ -200,22 +208,24 @@ static size_t latent_attention_lds(int R, int rot) {
 
 using namespace lc;
 
-// proj [T, ld]: [H x (dim | rot) | R | rot | ...]; cache [slots, R + rot]; qa [T, H, R + rot].
+// q [T, ldq]: [H x (dim | rot) | ...]; kv [T, ld]: [R | rot | ...]; cache [slots, R + rot]; qa [T, H, R + rot].
 // table: float32 [positions, rd] (cosines, then sines) or null; rd <= rot.
-LC_API int lc_latent_prepare(const void* proj, int dt, long long ld, int T, int H, int dim, int rot, int R,
+LC_API int lc_latent_prepare(const void* q, long long ldq, const void* proj, int dt, long long ld, int T, int H,
+                             int dim, int rot, int R,
                              const float* w, float eps, const int* positions, const float* table, int rd,
                              int interleaved, void* cache, const int* slots, void* qa, hipStream_t stream) {
     LC_CHECK(T >= 0 && H > 0 && dim >= 0 && rot >= 0 && R > 0, "latent prepare: bad sizes");
     if (T == 0) return 0;
-    LC_CHECK(proj && w && qa, "latent prepare: null pointer");
-    LC_CHECK(ld >= (long long)H * (dim + rot) + R + rot, "latent prepare: rows of %lld entries are too short", ld);
+    LC_CHECK(q && proj && w && qa, "latent prepare: null pointer");
+    LC_CHECK(ld >= (long long)R + rot && ldq >= (long long)H * (dim + rot),
+             "latent prepare: rows of %lld and %lld entries are too short", ldq, ld);
     LC_CHECK(!table || (positions && rd > 0 && rd % 2 == 0 && rd <= rot), "latent prepare: %d rotated entries in a part of %d", rd, rot);
     LC_CHECK((cache == nullptr) == (slots == nullptr), "latent prepare: cache and slots come together");
     if (dt == DT_F32)
-        latent_prepare_kernel<float><<<T, LA_THREADS, 0, stream>>>((const float*)proj, ld, H, dim, rot, R, w, eps, positions,
+        latent_prepare_kernel<float><<<T, LA_THREADS, 0, stream>>>((const float*)q, ldq, (const float*)proj, ld, H, dim, rot, R, w, eps, positions,
                                                                   table, rd, interleaved, (float*)cache, slots, (float*)qa);
     else if (dt == DT_BF16)
-        latent_prepare_kernel<bf16><<<T, LA_THREADS, 0, stream>>>((const bf16*)proj, ld, H, dim, rot, R, w, eps, positions,
+        latent_prepare_kernel<bf16><<<T, LA_THREADS, 0, stream>>>((const bf16*)q, ldq, (const bf16*)proj, ld, H, dim, rot, R, w, eps, positions,
                                                                  table, rd, interleaved, (bf16*)cache, slots, (bf16*)qa);
     else
         LC_CHECK(false, "latent prepare: unknown dtype %d", dt);
@@ -226,7 +236,8 @@ LC_API int lc_latent_prepare(const void* proj, int dt, long long ld, int T, int 
 // qa [T, H, R + rot], cache [slots, R + rot] -> out [T, H, R]
 LC_API int lc_latent_attention(const void* qa, int dt, int T, int H, int R, int rot, const void* cache,
                                const int* tok_req, const int* positions, const int* block_table, int max_blocks,
-                               int page_size, float scale, int window, void* out, hipStream_t stream) {
+                               int page_size, float scale, int window, const float* sink, void* out,
+                               hipStream_t stream) {
     LC_CHECK(T >= 0 && H > 0 && R > 0 && rot >= 0 && page_size > 0 && max_blocks > 0, "latent attention: bad sizes");
     if (T == 0) return 0;
     LC_CHECK(qa && cache && tok_req && positions && block_table && out, "latent attention: null pointer");
@@ -239,7 +250,7 @@ LC_API int lc_latent_attention(const void* qa, int dt, int T, int H, int R, int 
     const bool vec = (R + rot) % 4 == 0 && (uintptr_t)cache % 16 == 0;
 #define LC_LA_LAUNCH(TYPE, VEC)                                                                                   \
     latent_attention_kernel<TYPE, VEC><<<grid, LA_THREADS, lds, stream>>>((const TYPE*)qa, H, R, rot, (const TYPE*)cache, \
-        tok_req, positions, block_table, max_blocks, page_size, scale, window, (TYPE*)out)
+        tok_req, positions, block_table, max_blocks, page_size, scale, window, sink, (TYPE*)out)
     if (dt == DT_F32) {
         if (vec) LC_LA_LAUNCH(float, true); else LC_LA_LAUNCH(float, false);
     } else if (dt == DT_BF16) {

@@ -40,8 +40,8 @@ template <int NR, int KS>
 __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     const bf16* __restrict__ qa, int H, int R, int rot, const bf16* __restrict__ cache,
     const int* __restrict__ tiles, const int* __restrict__ block_table, int max_blocks, int page_size,
-    float scale, int window, bf16* __restrict__ out, int splits, float* __restrict__ part_o,
-    float* __restrict__ part_ml) {
+    float scale, int window, const float* __restrict__ sink, bf16* __restrict__ out, int splits,
+    float* __restrict__ part_o, float* __restrict__ part_ml) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const int Dk = R + rot, Dp = KS * 32;
     const int kstride = Dp + LM_KPAD;                       // bf16 a staged row
@@ -253,7 +253,15 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
     // the lane holds the entries 16 d + 4 g + r of its column
     const size_t qi = (size_t)(t0 + q_tok) * H + q_head;
     if (splits == 1) {
-        const float inv = 1.f / l_run;
+        float inv = 1.f / l_run;
+        if (sink) {
+            // one more term in the denominator: exp(sink), a key with that score and no value (the
+            // maxima are in units of log 2)
+            const float s2 = sink[q_head] * 1.4426950408889634f;
+            const float m_all = fmaxf(m_run, s2);
+            const float keep = __builtin_amdgcn_exp2f(m_run - m_all);
+            inv = keep / fmaf(l_run, keep, __builtin_amdgcn_exp2f(s2 - m_all));
+        }
 #pragma unroll
         for (int d = 0; d < NH; ++d)
             if ((half * NH + d) * 16 < R) {
@@ -277,18 +285,21 @@ __global__ __launch_bounds__(LM_THREADS) void latent_attention_bf16_kernel(
 
 // One workgroup per (token, head): the shares' sums, taken in from the first.
 __global__ void latent_attention_join_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                             int splits, int R, bf16* __restrict__ out) {
+                                             int splits, int R, int H, const float* __restrict__ sink,
+                                             bf16* __restrict__ out) {
     __shared__ float weight[64];
     __shared__ float total;
     const size_t qi = blockIdx.x;
     if (threadIdx.x < 64) {
         const int z = threadIdx.x;
         const float m = z < splits ? part_ml[(qi * splits + z) * 2] : -INFINITY;
-        const float M = wave_max(m);
+        // the head's sink counts as one more share: maximum sink, sum 1, no row
+        const float s2 = sink ? sink[qi % H] * 1.4426950408889634f : -INFINITY;
+        const float M = fmaxf(wave_max(m), s2);
         const float w = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);     // the maxima are in units of log 2
         weight[z] = w;
         const float L = wave_sum(z < splits ? part_ml[(qi * splits + z) * 2 + 1] * w : 0.f);
-        if (z == 0) total = L;
+        if (z == 0) total = L + (sink ? __builtin_amdgcn_exp2f(s2 - M) : 0.f);
     }
     __syncthreads();
     const float inv = 1.f / total;
@@ -336,8 +347,8 @@ LC_API int lc_latent_bf16_splits(int workgroups, int max_keys) {
 // splits 2] float32.
 LC_API int lc_latent_attention_bf16(const void* qa, int T, int H, int R, int rot, const void* cache, const int* tiles,
                                     int num_tiles, int any_portion, const int* block_table, int max_blocks,
-                                    int page_size, float scale, int window, void* out, int splits, float* part_o,
-                                    float* part_ml, hipStream_t stream) {
+                                    int page_size, float scale, int window, const float* sink, void* out, int splits,
+                                    float* part_o, float* part_ml, hipStream_t stream) {
     int nr = 0, ks = 0;
     LC_CHECK(shape_of(R, rot, &nr, &ks), "latent attention: the matrix-core kernel does not take a latent of %d + %d", R, rot);
     LC_CHECK(T >= 0 && H > 0 && num_tiles >= 0 && page_size > 0 && max_blocks > 0 && splits >= 1 && splits <= 65535,
@@ -358,7 +369,7 @@ LC_API int lc_latent_attention_bf16(const void* qa, int T, int H, int R, int rot
                      "latent attention: %zu bytes of LDS refused", lds);                                           \
         latent_attention_bf16_kernel<NR, KS><<<grid, LM_THREADS, lds, stream>>>(                                    \
             (const bf16*)qa, H, R, rot, (const bf16*)cache, tiles, block_table, max_blocks, page_size, scale, window, \
-            (bf16*)out, splits, part_o, part_ml);                                                                  \
+            sink, (bf16*)out, splits, part_o, part_ml);                                                               \
     } while (0)
     if (nr == 4) LC_LM_LAUNCH(4, 4);
     else if (nr == 8) LC_LM_LAUNCH(8, 8);
@@ -367,7 +378,7 @@ LC_API int lc_latent_attention_bf16(const void* qa, int T, int H, int R, int rot
 #undef LC_LM_LAUNCH
     LC_LAUNCH_CHECK("latent_attention_bf16");
     if (splits > 1) {
-        latent_attention_join_kernel<<<T * H, 256, 0, stream>>>(part_o, part_ml, splits, R, (bf16*)out);
+        latent_attention_join_kernel<<<T * H, 256, 0, stream>>>(part_o, part_ml, splits, R, H, sink, (bf16*)out);
         LC_LAUNCH_CHECK("latent_attention_join");
     }
     return 0;

@@ -104,6 +104,94 @@ __global__ __launch_bounds__(kWave) void moe_route_logits_kernel(const float* __
     if (lane < top) weights[(size_t)t * top + lane] = mine / picked_sum;
 }
 
+// One wave per token: scores s = sigmoid(z); the choice goes by s + correction, the weights by s alone,
+// times `scale`.  With `groups` > 1 the experts form that many equal groups of neighbours; a group's
+// rank is the sum of its two largest choice scores (of its one, where a group is one expert), and only
+// the experts of the `keep` best groups can be chosen: the others leave the contest whatever their
+// score.  The lower index wins every tie, among groups and among experts.
+__global__ __launch_bounds__(kWave) void moe_route_sigmoid_kernel(const float* __restrict__ logits,
+                                                                 const float* __restrict__ correction, int E,
+                                                                 int top, int groups, int keep, float scale,
+                                                                 int* __restrict__ ids, float* __restrict__ weights) {
+    __shared__ float choice_s[MOE_MAX_EXPERTS];
+    __shared__ float score_s[MOE_MAX_EXPERTS];
+    __shared__ float rank_s[MOE_MAX_EXPERTS];
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (size_t)t * E;
+    float c[MOE_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < MOE_PER_LANE; ++i) {
+        const int e = lane + kWave * i;
+        c[i] = -INFINITY;
+        if (e < E) {
+            const float s = 1.f / (1.f + expf(-z[e]));
+            score_s[e] = s;
+            c[i] = s + (correction ? correction[e] : 0.f);
+            choice_s[e] = c[i];
+        }
+    }
+    __syncthreads();
+    if (groups > 1) {
+        const int per = E / groups;
+        for (int g = lane; g < groups; g += kWave) {
+            float a = -INFINITY, b = -INFINITY;          // the largest and the second largest of the group
+            for (int e = g * per; e < (g + 1) * per; ++e) {
+                const float v = choice_s[e];
+                if (v > a) { b = a; a = v; }
+                else if (v > b) b = v;
+            }
+            rank_s[g] = per > 1 ? a + b : a;
+        }
+        __syncthreads();
+        // the `keep` best groups, one at a time; +infinity in place of its rank marks a kept group
+        for (int k = 0; k < keep; ++k) {
+            float best = -INFINITY;
+            int at = 0x7fffffff;
+            for (int g = lane; g < groups; g += kWave) {
+                const float v = rank_s[g];
+                if (v != INFINITY && (v > best || at == 0x7fffffff)) { best = v; at = g; }
+            }
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, kWave);
+                const int oa = __shfl_xor(at, off, kWave);
+                if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+            }
+            if (lane == 0 && at != 0x7fffffff) rank_s[at] = INFINITY;
+            __syncthreads();
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i) {
+            const int e = lane + kWave * i;
+            if (e < E && rank_s[e / per] != INFINITY) c[i] = -INFINITY;
+        }
+    }
+    // the `top` largest choice scores that are left (`gone`: taken already, or no expert at all)
+    bool gone[MOE_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < MOE_PER_LANE; ++i) gone[i] = lane + kWave * i >= E;
+    float mine = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i)
+            if (!gone[i] && (at == 0x7fffffff || c[i] > best)) { best = c[i]; at = lane + kWave * i; }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, kWave);
+            const int oa = __shfl_xor(at, off, kWave);
+            if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_PER_LANE; ++i)
+            if (lane + kWave * i == at) gone[i] = true;
+        if (lane == 0) ids[(size_t)t * top + k] = at;
+        if (lane == k) mine = score_s[at] * scale;
+    }
+    if (lane < top) weights[(size_t)t * top + lane] = mine;
+}
+
 // One workgroup: counts, the two running sums, and every pair's sorted row.
 __global__ __launch_bounds__(1024) void moe_lists_kernel(const int* __restrict__ ids, int n, int top, int E,
                                                          int tile, int* __restrict__ row_start,
@@ -245,5 +333,18 @@ LC_API int lc_moe_combine_shared(const float* y, const float* weights, const int
     else LC_CHECK(false, "moe combine: unknown dtypes %d, %d", dt, dt_shared);
 #undef LC_COMBINE
     LC_LAUNCH_CHECK("moe_combine_shared");
+    return 0;
+}
+
+// logits float32 [T, E], correction float32 [E] or null -> ids int32 [T, top], weights float32 [T, top]
+LC_API int lc_moe_route_sigmoid(const float* logits, const float* correction, int T, int E, int top, int groups,
+                                int keep, float scale, int* ids, float* weights, hipStream_t stream) {
+    LC_CHECK(T >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= kWave, "moe route: bad sizes E=%d top=%d", E, top);
+    LC_CHECK(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (E / groups),
+             "moe route: %d groups of which %d are kept do not hold %d choices among %d experts", groups, keep, top, E);
+    if (T == 0) return 0;
+    LC_CHECK(logits && ids && weights, "moe route: null pointer");
+    moe_route_sigmoid_kernel<<<T, kWave, 0, stream>>>(logits, correction, E, top, groups, keep, scale, ids, weights);
+    LC_LAUNCH_CHECK("moe_route_sigmoid");
     return 0;
 }

@@ -27,7 +27,7 @@ _ARG = {"p": ctypes.c_void_p, "i": ctypes.c_int, "f": ctypes.c_float, "q": ctype
 _SIGNATURES = {
     "lc_embedding": "ppipiiifp",
     "lc_rmsnorm": "ppppfpiiiipiip",
-    "lc_rmsnorm_act": "ppfpiiip",
+    "lc_rmsnorm_act": "pqpfpiiip",
     "lc_gemm_generic": "pipipiiiipp",
     "lc_gemm_bf16": "pppiiiiipp",
     "lc_gemm_bf16_supported": "iii",
@@ -71,18 +71,23 @@ _SIGNATURES = {
     "lc_sample_workspace": "i",
     "lc_feed_tokens": "pppiip",
     "lc_dynamic_tanh": "pppppfpiiiip",
-    "lc_stream_add": "ppipiip",
-    "lc_activation": "piiqp",
+    "lc_stream_add": "ppippiip",
+    "lc_activation": "piiffqp",
+    "lc_scale": "pfqp",
+    "lc_token_shift": "pippppppiip",
+    "lc_rms_shift": "ppipffppppppiiip",
     "lc_gemm_grouped": "piqqpipiqqiiiipppiiipqqp",
     "lc_gemm_grouped_fast": "i",
     "lc_gemm_grouped_takes_tile": "iii",
-    "lc_latent_prepare": "piqiiiiipfppiipppp",
-    "lc_latent_attention": "piiiiippppiifipp",
+    "lc_latent_prepare": "pqpiqiiiiipfppiipppp",
+    "lc_latent_attention": "piiiiippppiifippp",
     "lc_latent_bf16_supported": "ii",
     "lc_latent_bf16_splits": "ii",
-    "lc_latent_attention_bf16": "piiiippiipiifipippp",
+    "lc_latent_attention_bf16": "piiiippiipiifippippp",
     "lc_moe_max_experts": "",
     "lc_moe_route": "piiiifppp",
+    "lc_moe_route_sigmoid": "ppiiiiifppp",
+    "lc_lightning_prepare": "piiiiipppp",
     "lc_moe_lists": "piiiippppp",
     "lc_moe_combine": "pppiiipip",
     "lc_layer_norm": "ppippfpppfpiiiiip",
@@ -356,15 +361,23 @@ def rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
     return ScaledRows(out, parts, 1, float(eps), h, weight) if scaled else out
 
 
-def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """RMSNorm over the last dimension of an activation tensor."""
+def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float, column: Optional[int] = None) -> torch.Tensor:
+    """RMSNorm over the last dimension of an activation tensor.  With ``column``: over the columns
+    ``column`` .. ``column`` + len(weight) of the 2-D ``x`` alone -> [rows, len(weight)]."""
     _need(x, "rmsnorm_act x")
     _need(weight, "rmsnorm_act weight", torch.float32, 1)
-    n = x.shape[-1]
-    if weight.shape[0] != n:
-        raise KernelError(f"rmsnorm_act: weight has {weight.shape[0]} entries for rows of {n}")
+    n = weight.shape[0]
+    if column is not None:
+        if x.dim() != 2 or column < 0 or column + n > x.shape[1]:
+            raise KernelError(f"rmsnorm_act: columns {column}..{column + n} of {tuple(x.shape)}")
+        out = torch.empty((x.shape[0], n), dtype=x.dtype, device=x.device)
+        _call("lc_rmsnorm_act", ctypes.c_void_p(x.data_ptr() + column * x.element_size()), x.shape[1], _ptr(weight),
+              _c_float(eps), _ptr(out), _c_int(_dt(x)), _c_int(x.shape[0]), _c_int(n), _stream())
+        return out
+    if x.shape[-1] != n:
+        raise KernelError(f"rmsnorm_act: weight has {weight.shape[0]} entries for rows of {x.shape[-1]}")
     out = torch.empty_like(x)
-    _call("lc_rmsnorm_act", _ptr(x), _ptr(weight), _c_float(eps), _ptr(out), _c_int(_dt(x)),
+    _call("lc_rmsnorm_act", _ptr(x), n, _ptr(weight), _c_float(eps), _ptr(out), _c_int(_dt(x)),
           _c_int(x.numel() // n), _c_int(n), _stream())
     return out
 
@@ -893,8 +906,9 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------------------ other norms, other feed-forwards
-ACTIVATIONS = {"gelu_tanh": 1, "relu_squared": 2}
-_EPILOGUE_GATE = 3
+ACTIVATIONS = {"gelu_tanh": 1, "relu_squared": 2, "xielu": 5}     # xielu takes two numbers (``params``)
+_EPILOGUE_GATE, _EPILOGUE_GROUP_GATE = 3, 4
+_EPILOGUES = {"gelu_tanh": 1, "relu_squared": 2}                    # what a grouped product can apply itself
 
 
 def dynamic_tanh(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor,
@@ -921,8 +935,10 @@ def dynamic_tanh(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.T
     return out
 
 
-def stream_add(h: torch.Tensor, delta: Optional[torch.Tensor], vector: torch.Tensor) -> None:
-    """``h[t] += delta[t] + vector`` for every row of the float32 residual stream ``h`` [T, n]."""
+def stream_add(h: torch.Tensor, delta: Optional[torch.Tensor], vector: torch.Tensor,
+               more: Optional[torch.Tensor] = None) -> None:
+    """``h[t] += delta[t] (+ more[t]) + vector`` for every row of the float32 residual stream ``h`` [T, n];
+    ``more`` float32 [T, n]."""
     _need(h, "stream_add h", torch.float32, 2)
     _need(vector, "stream_add vector", torch.float32, 1)
     T, n = h.shape
@@ -932,20 +948,77 @@ def stream_add(h: torch.Tensor, delta: Optional[torch.Tensor], vector: torch.Ten
         _need(delta, "stream_add delta", None, 2)
         if tuple(delta.shape) != (T, n):
             raise KernelError(f"stream_add: delta {tuple(delta.shape)} does not match h {(T, n)}")
-    _call("lc_stream_add", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, _ptr(vector), T, n,
-          _stream())
+    if more is not None:
+        _need(more, "stream_add more", torch.float32, 2)
+        if tuple(more.shape) != (T, n):
+            raise KernelError(f"stream_add: more {tuple(more.shape)} does not match h {(T, n)}")
+    _call("lc_stream_add", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, _ptr(more), _ptr(vector),
+          T, n, _stream())
 
 
-def activation(x: torch.Tensor, kind: str) -> torch.Tensor:
-    """``x`` through one of ACTIVATIONS, in place; returns ``x``."""
+def activation(x: torch.Tensor, kind: str, params=(0.0, 0.0)) -> torch.Tensor:
+    """``x`` through one of ACTIVATIONS, in place; returns ``x``.  ``params``: the two numbers of "xielu"
+    (z > 0: a z^2 + z/2; z <= 0: b (e^z - 1 - z) + z/2)."""
     _need(x, "activation x")
-    _call("lc_activation", _ptr(x), _dt(x), ACTIVATIONS[kind], x.numel(), _stream())
+    _call("lc_activation", _ptr(x), _dt(x), ACTIVATIONS[kind], float(params[0]), float(params[1]), x.numel(), _stream())
     return x
 
 
-def gemm_act(x, w: torch.Tensor, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
+def gemm_act(x, w: torch.Tensor, kind: str, out_dtype: torch.dtype, params=(0.0, 0.0)) -> torch.Tensor:
     """``act(x . w^T)``: the first product of a two-matrix feed-forward with its activation."""
-    return activation(gemm(x, w, out_dtype), kind)
+    return activation(gemm(x, w, out_dtype), kind, params)
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """float32 ``x`` times ``factor``, in place; returns ``x``."""
+    _need(x, "scale_ x", torch.float32)
+    _call("lc_scale", _ptr(x), float(factor), x.numel(), _stream())
+    return x
+
+
+def _check_shift(T: int, n: int, mix, state, tok_req, q_offsets, slot_ids, what: str) -> None:
+    _need(mix, f"{what} mix", torch.float32, 1)
+    _need(state, f"{what} state", torch.float32, 2)
+    _need(tok_req, "tok_req", torch.int32, 1)
+    _need(q_offsets, "q_offsets", torch.int32, 1)
+    _need(slot_ids, "slot_ids", torch.int32, 1)
+    if mix.shape[0] != n or state.shape[1] != n or tok_req.shape[0] != T or q_offsets.shape[0] != slot_ids.shape[0] + 1:
+        raise KernelError(f"{what}: mix, state or the request lists do not fit {T} rows of {n}")
+
+
+def token_shift(x: torch.Tensor, mix: torch.Tensor, state: torch.Tensor, tok_req: torch.Tensor,
+                q_offsets: torch.Tensor, slot_ids: torch.Tensor) -> torch.Tensor:
+    """``y[t] = x[t] + (x[t - 1] - x[t]) * mix`` within every request; the row before a request's first token
+    of the step is ``state[slot]`` (float32 [slots, n]), which then takes the request's last row."""
+    _need(x, "token_shift x", None, 2)
+    T, n = x.shape
+    _check_shift(T, n, mix, state, tok_req, q_offsets, slot_ids, "token_shift")
+    y = torch.empty_like(x)
+    _call("lc_token_shift", _ptr(x), _dt(x), _ptr(mix), _ptr(state), _ptr(tok_req), _ptr(q_offsets), _ptr(slot_ids),
+          _ptr(y), T, n, _stream())
+    return y
+
+
+def rms_shift(h: torch.Tensor, delta, gain: float, eps: float, mix: torch.Tensor, state: torch.Tensor,
+              tok_req: torch.Tensor, q_offsets: torch.Tensor, slot_ids: torch.Tensor, out_dtype: torch.dtype):
+    """The residual addition, an RMS norm with one number as its weight and the token shift in one kernel:
+    v = h + delta; u = v / sqrt(mean(v^2) + eps) * gain; y[t] = u[t] + (u[t - 1] - u[t]) * mix, the row before
+    a request's first token of the step being ``state[slot]``, which then takes the request's last u (float32).
+    Returns (v float32 [T, n], a new tensor; y [T, n] of ``out_dtype``)."""
+    _need(h, "rms_shift h", torch.float32, 2)
+    T, n = h.shape
+    delta = value(delta)
+    if delta is not None:
+        _need(delta, "rms_shift delta", None, 2)
+        if tuple(delta.shape) != (T, n):
+            raise KernelError(f"rms_shift: delta {tuple(delta.shape)} does not match h {(T, n)}")
+    _check_shift(T, n, mix, state, tok_req, q_offsets, slot_ids, "rms_shift")
+    h_out = torch.empty_like(h)
+    y = torch.empty((T, n), dtype=out_dtype, device=h.device)
+    _call("lc_rms_shift", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, _ptr(h_out), float(gain),
+          float(eps), _ptr(mix), _ptr(state), _ptr(tok_req), _ptr(q_offsets), _ptr(slot_ids), _ptr(y), _dt(y), T, n,
+          _stream())
+    return h_out, y
 
 
 @dataclass
@@ -981,21 +1054,22 @@ def _grouped_tile(rows: int, N: int, groups: int, x: torch.Tensor, w: torch.Tens
 
 
 def grouped_gemm(x: Strided, w: torch.Tensor, out: Strided, rows: int, gate: Optional[Strided] = None,
-                 activation: Optional[str] = None) -> None:
+                 activation: Optional[str] = None, gate_per_group: bool = False) -> None:
     """For every group g: ``out_g = x_g . w[g]^T`` over the first ``rows`` rows, with ``w`` [G, N, K], x_g
     the K columns of group g of ``x`` and out_g the N columns of group g of ``out`` (a product per
     head over all tokens, in one launch).  With ``gate``: the result times sigmoid of the gate's
-    entry at the same row and column of its group.  True 32-bit arithmetic whatever the types."""
+    entry at the same row and column of its group; ``gate_per_group``: the gate has ONE entry per row and
+    group (a number per token and head).  True 32-bit arithmetic whatever the types."""
     _need(w, "grouped_gemm w", None, 3)
     G, N, K = w.shape
     _check_strided(x, "grouped_gemm x", rows, G, K)
     _check_strided(out, "grouped_gemm out", rows, G, N)
-    epilogue = ACTIVATIONS[activation] if activation else 0
+    epilogue = _EPILOGUES[activation] if activation else 0
     if gate is not None:
         if activation:
             raise KernelError("grouped_gemm: a gate or an activation, not both")
-        _check_strided(gate, "grouped_gemm gate", rows, G, N, x.tensor.dtype)
-        epilogue = _EPILOGUE_GATE
+        _check_strided(gate, "grouped_gemm gate", rows, G, 1 if gate_per_group else N, x.tensor.dtype)
+        epilogue = _EPILOGUE_GROUP_GATE if gate_per_group else _EPILOGUE_GATE
     if rows == 0:
         return
     _call("lc_gemm_grouped", x.pointer(), _dt(x.tensor), x.tensor.shape[1], x.group, _ptr(w), _dt(w),
@@ -1013,7 +1087,8 @@ def grouped_gemm_matrix_cores(on: bool) -> bool:
 # ------------------------------------------------------------------------------ latent attention
 def latent_prepare(proj: torch.Tensor, heads: int, dim: int, rot: int, rank: int, norm_weight: torch.Tensor,
                    eps: float, positions: torch.Tensor, rope_table: Optional[torch.Tensor], pairing: str,
-                   cache: torch.Tensor, slots: Optional[torch.Tensor], qa: torch.Tensor) -> None:
+                   cache: torch.Tensor, slots: Optional[torch.Tensor], qa: torch.Tensor,
+                   q: Optional[torch.Tensor] = None, kv_column: Optional[int] = None) -> None:
     """What latent attention does to a step's projections ``proj`` [T, heads (dim + rot) + rank + rot
     (+ more)] before it attends: the ``rank`` entries behind the q heads, divided by their root mean
     square and times ``norm_weight``, and the ``rot`` entries behind them, rotated at the token's
@@ -1021,16 +1096,25 @@ def latent_prepare(proj: torch.Tensor, heads: int, dim: int, rot: int, rank: int
     page size + offset; negative or None: no write); every head's ``rot`` query entries, rotated,
     go to ``qa`` [T, heads (rank + rot)] behind the head's ``rank`` entries (which a product fills).
     ``rope_table`` [positions, rd] holds cosines, then sines; the first rd entries of a part are
-    rotated, as pairs (2i, 2i + 1) (``pairing`` "interleaved") or (i, i + rd/2) ("half")."""
+    rotated, as pairs (2i, 2i + 1) (``pairing`` "interleaved") or (i, i + rd/2) ("half").
+    With ``q`` [T, heads (dim + rot)] the heads' queries come from that tensor (a product of their own) and
+    ``proj`` holds [rank | rot | ...] from ``kv_column`` on."""
     _need(proj, "latent_prepare proj", None, 2)
     T = proj.shape[0]
+    if q is None:
+        q, kv_column = proj, heads * (dim + rot)
+    else:
+        _need(q, "latent_prepare q", proj.dtype, 2)
+        kv_column = int(kv_column or 0)
+        if q.shape[0] != T or q.shape[1] < heads * (dim + rot):
+            raise KernelError(f"latent_prepare: q {tuple(q.shape)} does not hold {heads} heads of {dim} + {rot}")
     _need(norm_weight, "latent norm weight", torch.float32, 1)
     if norm_weight.shape[0] != rank:
         raise KernelError(f"latent_prepare: norm weight has {norm_weight.shape[0]} entries for a latent of {rank}")
     _need(qa, "latent_prepare qa", proj.dtype, 2)
     if tuple(qa.shape) != (T, heads * (rank + rot)):
         raise KernelError(f"latent_prepare: qa {tuple(qa.shape)} is not [{T}, {heads * (rank + rot)}]")
-    if proj.shape[1] < heads * (dim + rot) + rank + rot:
+    if proj.shape[1] < kv_column + rank + rot:
         raise KernelError(f"latent_prepare: rows of {proj.shape[1]} entries are too short")
     rd = 0
     if rope_table is not None and rot:
@@ -1046,7 +1130,8 @@ def latent_prepare(proj: torch.Tensor, heads: int, dim: int, rot: int, rank: int
         _need(slots, "slots", torch.int32, 1)
         if cache.shape[2] != rank + rot or slots.shape[0] != T:
             raise KernelError(f"latent_prepare: cache rows of {cache.shape[2]} entries, expected {rank + rot}")
-    _call("lc_latent_prepare", _ptr(proj), _dt(proj), proj.shape[1], T, heads, dim, rot, rank, _ptr(norm_weight),
+    _call("lc_latent_prepare", _ptr(q), q.shape[1], ctypes.c_void_p(proj.data_ptr() + kv_column * proj.element_size()),
+          _dt(proj), proj.shape[1], T, heads, dim, rot, rank, _ptr(norm_weight),
           float(eps), _ptr(positions), _ptr(rope_table), rd, 1 if pairing == "interleaved" else 0,
           _ptr(cache if slots is not None else None), _ptr(slots), _ptr(qa), _stream())
 
@@ -1089,12 +1174,18 @@ def plan_latent_attention(layout):
 
 def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req: torch.Tensor,
                      positions: torch.Tensor, block_table: torch.Tensor, cache: torch.Tensor, page_size: int,
-                     scale: float, window: int = 0, plan=None, max_ctx: int = 0) -> torch.Tensor:
+                     scale: float, window: int = 0, plan=None, max_ctx: int = 0,
+                     sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention in the latent's space: queries ``qa`` [T, heads (rank + rot)] against the cached
     rows [c | k_r] of the token's request (``cache`` [pages, page, rank + rot], ``block_table`` [R,
     blocks]), weights softmax(q . row * scale) over the positions j <= p (and j > p - window), result
-    the weighted sum of the rows' first ``rank`` entries -> [T, heads rank]."""
+    the weighted sum of the rows' first ``rank`` entries -> [T, heads rank].  ``sink`` float32 [heads]: the
+    softmax's denominator of head h holds one more term, exp(sink[h]) (not scaled, no row)."""
     _need(qa, "latent_attention qa", None, 2)
+    if sink is not None:
+        _need(sink, "latent_attention sink", torch.float32, 1)
+        if sink.shape[0] != heads:
+            raise KernelError(f"latent_attention: {sink.shape[0]} sinks for {heads} heads")
     _need(cache, "latent cache", qa.dtype, 3)
     T = qa.shape[0]
     if qa.shape[1] != heads * (rank + rot) or cache.shape[2] != rank + rot or cache.shape[1] != page_size:
@@ -1122,7 +1213,7 @@ def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req:
             part_ml = torch.empty((T * heads * splits * 2,), dtype=torch.float32, device=qa.device)
         _call("lc_latent_attention_bf16", _ptr(qa), T, heads, rank, rot, _ptr(cache), _ptr(tiles), tiles.shape[0],
               1 if any_portion else 0, _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
-              _ptr(out), splits, _ptr(part_o), _ptr(part_ml), _stream())
+              _ptr(sink), _ptr(out), splits, _ptr(part_o), _ptr(part_ml), _stream())
         return out
     if qa.dtype == torch.bfloat16 and plan is not None and _latent_fast.on and rank * heads >= 1024:
         _say_once(("latent attention", rank, rot),
@@ -1131,7 +1222,7 @@ def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req:
                   "kernel runs, correct and many times slower")
     _call("lc_latent_attention", _ptr(qa), _dt(qa), T, heads, rank, rot, _ptr(cache), _ptr(tok_req),
           _ptr(positions), _ptr(block_table), block_table.shape[1], page_size, float(scale), int(window),
-          _ptr(out), _stream())
+          _ptr(sink), _ptr(out), _stream())
     return out
 
 
@@ -1176,6 +1267,32 @@ def moe_route(logits: torch.Tensor, top: int, renormalise: bool = True, eps: flo
     return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, tile, (T * top) // tile + E)
 
 
+def moe_route_sigmoid(logits: torch.Tensor, top: int, correction: Optional[torch.Tensor] = None, groups: int = 1,
+                      keep: int = 1, scale: float = 1.0, large_tiles: bool = False) -> Routing:
+    """As :func:`moe_route`, with scores s = sigmoid(logits): the ``top`` largest of s + ``correction`` [E] are
+    chosen (the lower index wins a tie) and weigh s * ``scale``, not renormalised.  ``groups`` > 1: the experts
+    form that many equal groups of neighbours, a group ranks by the sum of its two largest s + correction, and
+    only experts of the ``keep`` best groups can be chosen."""
+    _need(logits, "router logits", torch.float32, 2)
+    T, E = logits.shape
+    if correction is not None:
+        _need(correction, "router correction", torch.float32, 1)
+        if correction.shape[0] != E:
+            raise KernelError(f"moe_route_sigmoid: a correction of {correction.shape[0]} entries for {E} experts")
+    dev = logits.device
+    ids = torch.empty((T, top), dtype=torch.int32, device=dev)
+    weights = torch.empty((T, top), dtype=torch.float32, device=dev)
+    _call("lc_moe_route_sigmoid", _ptr(logits), _ptr(correction), T, E, top, int(groups), int(keep), float(scale),
+          _ptr(ids), _ptr(weights), _stream())
+    tile = 16 if T * top <= 16 * E else 128 if (large_tiles and T * top >= 192 * E) else 64
+    lists = torch.empty((2 * (E + 1) + 2 * T * top,), dtype=torch.int32, device=dev)
+    row_start, tile_start = lists[:E + 1], lists[E + 1:2 * (E + 1)]
+    sorted_token, entry_row = lists[2 * (E + 1):2 * (E + 1) + T * top], lists[2 * (E + 1) + T * top:]
+    _call("lc_moe_lists", _ptr(ids), T, top, E, tile, _ptr(row_start), _ptr(tile_start), _ptr(sorted_token),
+          _ptr(entry_row), _stream())
+    return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, tile, (T * top) // tile + E)
+
+
 def moe_large_tiles(x_dtype: torch.dtype, up: torch.Tensor, down: torch.Tensor) -> bool:
     """Whether both of the experts' products (weights ``up`` [E, I, H], ``down`` [E, H, I]) can run in tiles
     of 128 rows: bfloat16 operands whose rows are whole 16-byte pieces, 128 columns at least."""
@@ -1201,7 +1318,7 @@ def moe_experts(x: torch.Tensor, w: torch.Tensor, routing: Routing, out_dtype: t
     if rows:
         _call("lc_gemm_grouped", _ptr(x), _dt(x), K, 0, _ptr(w), _dt(w), _ptr(out), _dt(out), N, 0, rows, N, K, E,
               _ptr(routing.sorted_token if gather else None), _ptr(routing.row_start), _ptr(routing.tile_start),
-              routing.max_tiles, routing.tile, ACTIVATIONS[activation] if activation else 0,
+              routing.max_tiles, routing.tile, _EPILOGUES[activation] if activation else 0,
               None, 0, 0, _stream())
     return out
 
@@ -1598,3 +1715,22 @@ def moe_combine_shared(y: torch.Tensor, routing: Routing, shared: torch.Tensor, 
         _call("lc_moe_combine_shared", _ptr(y), _ptr(routing.weights), _ptr(routing.entry_row), T, top, n,
               _ptr(shared), _dt(shared), _ptr(gates), gates.shape[1], gate_column, _ptr(out), _dt(out), _stream())
     return out
+
+
+# ------------------------------------------------------------------------------ lightning attention
+def lightning_prepare(proj: torch.Tensor, heads: int, key_dim: int, value_dim: int, decay: torch.Tensor):
+    """The scan's inputs of lightning attention from the float32 projections ``proj`` [T, >= heads (2 key_dim
+    + value_dim)]: columns q | k | v.  Returns ``coef`` float32 [5, T, heads key_dim] (decay = ``decay``[head]
+    in every channel, probe = removal = 0, write = silu(k), read = silu(q)) and ``v`` = silu(v) float32
+    [T, heads value_dim]."""
+    _need(proj, "lightning proj", torch.float32, 2)
+    _need(decay, "lightning decay", torch.float32, 1)
+    T = proj.shape[0]
+    if proj.shape[1] < heads * (2 * key_dim + value_dim) or decay.shape[0] != heads:
+        raise KernelError(f"lightning_prepare: proj {tuple(proj.shape)} or decay do not fit {heads} heads")
+    coef = torch.empty((5, T, heads * key_dim), dtype=torch.float32, device=proj.device)
+    v = torch.empty((T, heads * value_dim), dtype=torch.float32, device=proj.device)
+    if T:
+        _call("lc_lightning_prepare", _ptr(proj), proj.shape[1], T, heads, key_dim, value_dim, _ptr(decay), _ptr(coef),
+              _ptr(v), _stream())
+    return coef, v

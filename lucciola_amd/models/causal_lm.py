@@ -85,15 +85,22 @@ def _end_parts(spec: ModelSpec):
     return embedding, head, head_names
 
 
+def _embedding_name(spec: ModelSpec, logical: str) -> str:
+    """The checkpoint name of one of the embedding's tensors: the table's is ``embedding_name``."""
+    if logical == "weight":
+        return spec.embedding_name
+    if logical not in (spec.embedding_names or {}):
+        raise KeyError(f"the embedding's tensor '{logical}' has no checkpoint name")
+    return spec.embedding_names[logical]
+
+
 def declared_tensors(spec: ModelSpec) -> Dict[str, ParamDecl]:
     """Every tensor a model of this spec wants, by checkpoint name."""
     spec.validate()
     embedding, head, head_names = _end_parts(spec)
     out: Dict[str, ParamDecl] = {}
     for logical, decl in embedding.declare().items():
-        if logical != "weight":
-            raise KeyError(f"the embedding's tensor '{logical}' has no checkpoint name")
-        out[spec.embedding_name] = decl
+        out[_embedding_name(spec, logical)] = decl
     for layer in spec.layers:
         out.update(_LayerParts(layer).declared())
     for i, entry in enumerate(spec.run_order):
@@ -127,7 +134,8 @@ class CausalLM:
         for line in self.load_notices:
             print(f"[lucciola_amd] {line}", file=sys.stderr, flush=True)
         self.embed, self.head_part, head_names = _end_parts(spec)
-        self.embed.bind({"weight": tensors[spec.embedding_name]}, self.ctx)
+        self.embed.bind({logical: tensors[_embedding_name(spec, logical)] for logical in self.embed.declare()},
+                        self.ctx)
         self.head_part.bind({logical: tensors[head_names[logical]]
                              for logical in self.head_part.declare()}, self.ctx,
                             shared=self.embed.table())
@@ -143,6 +151,8 @@ class CausalLM:
                 step = build_part(STREAM_STEPS, entry.before)
                 step.bind({logical: tensors[entry.before_names[logical]] for logical in step.declare()}, self.ctx)
                 self.before[index] = step
+        # a step that adds the stream as the embedding left it needs that kept aside
+        self.keeps_origin = any(getattr(step, "needs_origin", False) for step in self.before.values())
         self.final_norm = build_part(NORMS, spec.final_norm)
         self.final_norm.bind({logical: tensors[name]
                               for logical, name in spec.final_norm_names.items()}, self.ctx)
@@ -216,6 +226,12 @@ class CausalLM:
             stream = ResidualStream(self.embed.forward(batch.token_ids, batch.positions))
         else:
             stream = ResidualStream(self.embed.forward(batch.token_ids))
+        if self.keeps_origin:
+            # the stream itself is updated in place from here on: the embedding's output once more
+            if getattr(self.embed, "takes_positions", False):
+                stream.origin = self.embed.forward(batch.token_ids, batch.positions)
+            else:
+                stream.origin = self.embed.forward(batch.token_ids)
         for index, entry in enumerate(self.spec.run_order):
             if index in self.before:
                 self.before[index].forward(stream)

@@ -54,6 +54,7 @@ class ResidualStream:
     def __init__(self, h: torch.Tensor):
         self.h = h
         self.pending = None      # a tensor [T, H] or an ops.PendingProduct
+        self.origin = None       # the stream as the embedding left it, where a stream step asks for it
 
 
 class Part:

@@ -48,6 +48,52 @@ class PreNormMixerBlock:
         stream.pending = self.mixer.forward(x, site)
 
 
+def _caching_index(parts, part) -> int:
+    """Which of the site's caches belongs to ``part``: a site's caches follow the layer's caching parts
+    in the order of the block's slots."""
+    return [p for p in parts if p.cache_need() is not None].index(part)
+
+
+@BLOCKS.register("prenorm_shift_residual")
+class PreNormShiftResidualBlock:
+    """The pre-norm residual arrangement with an input shift between the first norm and the mixer:
+    h += mixer(shift(norm(h))); h += feed_forward(norm(h)).  The shift keeps state of its own beside the
+    mixer's cache."""
+
+    slots = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm",
+             "feed_forward_norm": "norm", "mixer_shift": "input_shift"}
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, mixer_shift):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm, self.mixer_shift = mixer_norm, feed_forward_norm, mixer_shift
+        order = (mixer, feed_forward, mixer_norm, feed_forward_norm, mixer_shift)
+        self._mixer_at = _caching_index(order, mixer) if mixer.cache_need() is not None else None
+        self._shift_at = _caching_index(order, mixer_shift)
+
+    def forward(self, stream: ResidualStream, site) -> None:
+        x = self.mixer_shift.add_norm_shift(self.mixer_norm, stream, site.part(self._shift_at))
+        stream.pending = self.mixer.forward(x, site.part(self._mixer_at) if self._mixer_at is not None else site)
+        x = PreNormResidualBlock._normed(self.feed_forward_norm, self.feed_forward, stream)
+        stream.pending = self.feed_forward.forward(x)
+
+
+@BLOCKS.register("prenorm_shift_mixer")
+class PreNormShiftMixerBlock:
+    """The same without a feed-forward: h += mixer(shift(norm(h)))."""
+
+    slots = {"mixer": "mixer", "mixer_norm": "norm", "mixer_shift": "input_shift"}
+
+    def __init__(self, mixer, mixer_norm, mixer_shift):
+        self.mixer, self.mixer_norm, self.mixer_shift = mixer, mixer_norm, mixer_shift
+        order = (mixer, mixer_norm, mixer_shift)
+        self._mixer_at = _caching_index(order, mixer) if mixer.cache_need() is not None else None
+        self._shift_at = _caching_index(order, mixer_shift)
+
+    def forward(self, stream: ResidualStream, site) -> None:
+        x = self.mixer_shift.add_norm_shift(self.mixer_norm, stream, site.part(self._shift_at))
+        stream.pending = self.mixer.forward(x, site.part(self._mixer_at) if self._mixer_at is not None else site)
+
+
 def _post_normed(norm, branch):
     """The branch output behind its norm: left to the next kernel that adds to the stream where
     the norm can say so (``behind``), else normed now."""

@@ -48,6 +48,29 @@ class TokenEmbedding(Part):
         return ops.embedding(ids, self.weight, self.scale)
 
 
+@EMBEDDINGS.register("normed_token_embedding")
+class NormedTokenEmbedding(TokenEmbedding):
+    """The table's row divided by its root mean square (``eps`` inside the root) and times one learned
+    number (tensor ``norm``, a scalar); float32 arithmetic."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, eps: float, scale: float = 1.0):
+        super().__init__(vocab_size, hidden_size, scale)
+        self.params["eps"] = eps
+        self.eps = float(eps)
+        self.gain: Optional[torch.Tensor] = None
+
+    def declare(self) -> Dict[str, ParamDecl]:
+        return {"weight": ParamDecl((self.V, self.H)),
+                "norm": ParamDecl((), role="vector", init="ones_plus_normal")}
+
+    def bind(self, tensors, ctx: BuildContext) -> None:
+        super().bind(tensors, ctx)
+        self.gain = tensors["norm"].to(torch.float32).reshape(1).expand(self.H).contiguous()
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        return ops.rmsnorm(ops.embedding(ids, self.weight, self.scale), None, self.gain, self.eps, torch.float32)
+
+
 @EMBEDDINGS.register("sinusoid_token_embedding")
 class SinusoidTokenEmbedding(TokenEmbedding):
     """The table's row plus a position vector: entry 2i is sin(p f_i), entry 2i + 1 cos(p f_i),
@@ -76,9 +99,10 @@ class SinusoidTokenEmbedding(TokenEmbedding):
 class LinearHead(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
-        super().__init__(vocab_size=vocab_size, hidden_size=hidden_size, tied=tied)
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, scale: float = 1.0):
+        super().__init__(vocab_size=vocab_size, hidden_size=hidden_size, tied=tied, scale=scale)
         self.V, self.H, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+        self.scale = float(scale)           # the logits are the product times this number
         self.weight: Optional[torch.Tensor] = None
 
     def declare(self) -> Dict[str, ParamDecl]:
@@ -90,4 +114,5 @@ class LinearHead(Part):
             raise ValueError("linear_head: a tied head needs the embedding's table")
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.gemm(x, self.weight, torch.float32)
+        logits = ops.gemm(x, self.weight, torch.float32)
+        return logits if self.scale == 1.0 else ops.scale_(logits, self.scale)

@@ -4,7 +4,8 @@ product here: their weights are stacked at load.  The gate's activation is a par
 or "gelu_tanh", which takes a kernel of its own behind the product)."""
 from __future__ import annotations
 
-from typing import Dict
+import math
+from typing import Dict, Optional
 
 import torch
 
@@ -12,6 +13,10 @@ from ..config.registry import FEED_FORWARDS
 from ..kernels import ops
 from ..weights.loader import ParamDecl
 from .base import BuildContext, Part
+
+
+def _softplus(z: float) -> float:
+    return math.log1p(math.exp(-abs(z))) + max(z, 0.0)
 
 
 def stack_rows(tensors):
@@ -65,7 +70,9 @@ class GatedMLP(Part):
 @FEED_FORWARDS.register("mlp")
 class MLP(Part):
     """The plain two-matrix feed-forward ``down(act(up(x)))``, no biases.  ``activation``:
-    "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))) or "relu_squared"."""
+    "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))), "relu_squared", or "xielu": with two
+    learned numbers p, q (tensor ``act``), z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q))
+    (e^z - 1 - z) + z/2."""
 
     graph_safe = True
 
@@ -77,14 +84,22 @@ class MLP(Part):
         self.H, self.I, self.activation = int(hidden_size), int(intermediate_size), activation
 
     def declare(self) -> Dict[str, ParamDecl]:
-        return {"up": ParamDecl((self.I, self.H)), "down": ParamDecl((self.H, self.I))}
+        out = {"up": ParamDecl((self.I, self.H)), "down": ParamDecl((self.H, self.I))}
+        if self.activation == "xielu":
+            out["act"] = ParamDecl((2,), role="vector", init="normal")
+        return out
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self.up, self.down = tensors["up"], tensors["down"]
         self.dtype = ctx.dtype
+        self.act_params = (0.0, 0.0)
+        if self.activation == "xielu":
+            # the two numbers as the kernel takes them; read once, at load
+            p, q = (float(v) for v in tensors["act"].to(torch.float64).cpu())
+            self.act_params = (_softplus(p), 0.5 + _softplus(q))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        z = ops.gemm_act(x, self.up, self.activation, self.dtype)
+        z = ops.gemm_act(x, self.up, self.activation, self.dtype, self.act_params)
         return ops.gemm(z, self.down, self.dtype, defer=True)
 
 
@@ -93,7 +108,11 @@ class RoutedMLP(Part):
     """A mixture of small two-matrix feed-forwards.  The router's logits (float32) become
     scores over all experts (``scores``: "softmax"); each token keeps its ``top`` largest, whose
     scores, divided by their sum + ``renormalise_eps`` where ``renormalise``, weigh the experts'
-    outputs.  On the device the (token, expert) pairs are sorted by expert, and the two products
+    outputs.  With ``scores`` "sigmoid" the scores are sigmoids of the logits: the choice goes by
+    score + a learned correction per expert (tensor ``correction``, where ``correction``), the
+    weights by the plain scores times ``weight_scale``, never renormalised; with ``groups`` > 1 the
+    experts form that many equal groups of neighbours, a group ranks by the sum of its two largest
+    corrected scores, and only experts of the ``keep_groups`` best groups can be chosen.  On the device the (token, expert) pairs are sorted by expert, and the two products
     run once over the sorted rows, each tile of rows with its expert's matrix; nothing of it
     passes the host."""
 
@@ -101,21 +120,35 @@ class RoutedMLP(Part):
 
     def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int,
                  activation: str = "relu_squared", scores: str = "softmax", renormalise: bool = True,
-                 renormalise_eps: float = 1e-20):
+                 renormalise_eps: float = 1e-20, correction: bool = False, groups: int = 1, keep_groups: int = 1,
+                 weight_scale: float = 1.0):
         super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size, experts=experts,
                          top=top, activation=activation, scores=scores, renormalise=renormalise,
-                         renormalise_eps=renormalise_eps)
-        if activation not in ops.ACTIVATIONS:
+                         renormalise_eps=renormalise_eps, correction=correction, groups=groups,
+                         keep_groups=keep_groups, weight_scale=weight_scale)
+        if activation not in ("gelu_tanh", "relu_squared"):
             raise ValueError(f"routed_mlp: activation '{activation}' has no kernel")
-        if scores != "softmax":
-            raise ValueError(f"routed_mlp: scores '{scores}' have no kernel (softmax)")
+        if scores not in ("softmax", "sigmoid"):
+            raise ValueError(f"routed_mlp: scores '{scores}' have no kernel (softmax, sigmoid)")
         if not 1 <= int(top) <= int(experts):
             raise ValueError(f"routed_mlp: top {top} of {experts} experts")
+        self.scores, self.correction = scores, bool(correction)
+        self.groups, self.keep_groups, self.weight_scale = int(groups), int(keep_groups), float(weight_scale)
+        if scores == "softmax" and (correction or self.groups > 1 or self.weight_scale != 1.0):
+            raise ValueError("routed_mlp: a correction, groups and a weight scale go with sigmoid scores")
+        if scores == "sigmoid" and renormalise:
+            raise ValueError("routed_mlp: sigmoid scores are not renormalised")
+        if self.groups < 1 or int(experts) % self.groups or not 1 <= self.keep_groups <= self.groups \
+                or int(top) > self.keep_groups * (int(experts) // self.groups):
+            raise ValueError(f"routed_mlp: {self.groups} groups of which {self.keep_groups} are kept do not hold "
+                             f"{top} choices among {experts} experts")
         self.H, self.I, self.E, self.top = int(hidden_size), int(intermediate_size), int(experts), int(top)
         self.activation, self.renormalise, self.renormalise_eps = activation, bool(renormalise), float(renormalise_eps)
 
     def declare(self) -> Dict[str, ParamDecl]:
         out = {"router": ParamDecl((self.E, self.H))}
+        if self.correction:
+            out["correction"] = ParamDecl((self.E,), role="vector", init="normal")
         for k in range(self.E):
             out[f"experts.{k}.up"] = ParamDecl((self.I, self.H))
             out[f"experts.{k}.down"] = ParamDecl((self.H, self.I))
@@ -123,6 +156,8 @@ class RoutedMLP(Part):
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self.router = tensors["router"]
+        self.correction_vector: Optional[torch.Tensor] = (
+            tensors["correction"].to(torch.float32).contiguous() if self.correction else None)
         self.up = stack_rows([tensors[f"experts.{k}.up"] for k in range(self.E)]).view(self.E, self.I, self.H)
         self.down = stack_rows([tensors[f"experts.{k}.down"] for k in range(self.E)]).view(self.E, self.H, self.I)
         self.dtype = ctx.dtype
@@ -130,8 +165,12 @@ class RoutedMLP(Part):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = ops.gemm(x, self.router, torch.float32)
-        routing = ops.moe_route(logits, self.top, self.renormalise, self.renormalise_eps,
-                                large_tiles=self.large_tiles)
+        if self.scores == "sigmoid":
+            routing = ops.moe_route_sigmoid(logits, self.top, self.correction_vector, self.groups, self.keep_groups,
+                                            self.weight_scale, large_tiles=self.large_tiles)
+        else:
+            routing = ops.moe_route(logits, self.top, self.renormalise, self.renormalise_eps,
+                                    large_tiles=self.large_tiles)
         hidden = ops.moe_experts(x, self.up, routing, self.dtype, activation=self.activation, gather=True)
         y = ops.moe_experts(hidden, self.down, routing, torch.float32)
         return ops.moe_combine(y, routing, self.dtype)

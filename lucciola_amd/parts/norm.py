@@ -18,17 +18,24 @@ class RMSNorm(Part):
     graph_safe = True   # launches only kernels whose arguments stay put between steps
     offers_scaled_rows = True   # add_norm(stream, scaled=True) may return ops.ScaledRows
 
-    def __init__(self, size: int, eps: float):
-        super().__init__(size=size, eps=eps)
+    def __init__(self, size: int, eps: float, scalar: bool = False):
+        super().__init__(size=size, eps=eps, scalar=scalar)
         self.size, self.eps = int(size), float(eps)
+        # scalar: the learned weight is one number for all coordinates (``gain``); the kernels still
+        # get a vector, that number in every entry
+        self.scalar = bool(scalar)
+        self.gain: Optional[float] = None
         self.weight: Optional[torch.Tensor] = None
         self.dtype = None
 
     def declare(self) -> Dict[str, ParamDecl]:
-        return {"weight": ParamDecl((self.size,), role="vector", init="ones_plus_normal")}
+        return {"weight": ParamDecl(() if self.scalar else (self.size,), role="vector", init="ones_plus_normal")}
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self.weight = tensors["weight"]
+        if self.scalar:
+            self.gain = float(self.weight.to(torch.float32).item())     # a kernel argument; read once, at load
+            self.weight = self.weight.to(torch.float32).reshape(1).expand(self.size).contiguous()
         self.dtype = ctx.dtype
 
     def add_norm(self, stream: ResidualStream, scaled: bool = False):

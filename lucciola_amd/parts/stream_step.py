@@ -15,13 +15,15 @@ from .base import BuildContext, Part, ResidualStream
 class RowOffset(Part):
     """Adds row ``row`` of a learned table [rows, size] to every token's stream: the mark of a
     pass where a stack of layers runs several times.  The branch output that still waits is
-    added by the same kernel."""
+    added by the same kernel.  ``add_origin``: the stream as the embedding left it is added as
+    well (a pass that starts again from the tokens themselves)."""
 
     graph_safe = True
 
-    def __init__(self, size: int, rows: int, row: int):
-        super().__init__(size=size, rows=rows, row=row)
+    def __init__(self, size: int, rows: int, row: int, add_origin: bool = False):
+        super().__init__(size=size, rows=rows, row=row, add_origin=add_origin)
         self.size, self.rows, self.row = int(size), int(rows), int(row)
+        self.needs_origin = bool(add_origin)
         if not 0 <= self.row < self.rows:
             raise ValueError(f"row_offset: row {row} of a table of {rows}")
         self.vector = None
@@ -33,5 +35,8 @@ class RowOffset(Part):
         self.vector = tensors["table"][self.row].contiguous()
 
     def forward(self, stream: ResidualStream) -> None:
-        ops.stream_add(stream.h, ops.value(stream.pending), self.vector)
+        if self.needs_origin and stream.origin is None:
+            raise ValueError("row_offset: the stream's origin was not kept")
+        ops.stream_add(stream.h, ops.value(stream.pending), self.vector,
+                       more=stream.origin if self.needs_origin else None)
         stream.pending = None

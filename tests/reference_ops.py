@@ -29,8 +29,8 @@ def rmsnorm(h, delta, weight, eps, out_dtype, rows=None, scaled=False):   # neve
     return (v * inv * weight.to(F64)).to(out_dtype)
 
 
-def rmsnorm_act(x, weight, eps):
-    v = x.to(F64)
+def rmsnorm_act(x, weight, eps, column=None):
+    v = x.to(F64) if column is None else x[:, column:column + weight.shape[0]].to(F64)
     inv = torch.rsqrt((v * v).mean(dim=-1, keepdim=True) + eps)
     return (v * inv * weight.to(F64)).to(x.dtype)
 
@@ -134,13 +134,50 @@ def dynamic_tanh(h, delta, weight, bias, alpha, out_dtype, rows=None):
     return (torch.tanh(alpha * v) * weight.to(F64) + bias.to(F64)).to(out_dtype)
 
 
-def stream_add(h, delta, vector):
+def stream_add(h, delta, vector, more=None):
     if delta is not None:
         h += delta.to(torch.float32)
+    if more is not None:
+        h += more
     h += vector
 
 
-def _act(z, kind):
+def scale_(x, factor):
+    x *= factor
+    return x
+
+
+def _shift_rows(u, mix, state, q_offsets, slot_ids):
+    """u [T, n] float64 normed rows -> shifted rows; the state takes every request's last row."""
+    y = torch.empty_like(u)
+    starts, slots = q_offsets.tolist(), slot_ids.tolist()
+    for r, slot in enumerate(slots):
+        a, b = starts[r], starts[r + 1]
+        if b <= a:
+            continue
+        before = torch.cat([state[slot].to(F64)[None], u[a:b - 1]], dim=0)
+        y[a:b] = u[a:b] + (before - u[a:b]) * mix.to(F64)
+        state[slot] = u[b - 1].to(torch.float32)
+    return y
+
+
+def token_shift(x, mix, state, tok_req, q_offsets, slot_ids):
+    return _shift_rows(x.to(F64), mix, state, q_offsets, slot_ids).to(x.dtype)
+
+
+def rms_shift(h, delta, gain, eps, mix, state, tok_req, q_offsets, slot_ids, out_dtype):
+    v = h.clone()
+    if delta is not None:
+        v += delta.to(torch.float32)
+    v64 = v.to(F64)
+    u = v64 * torch.rsqrt((v64 * v64).mean(dim=-1, keepdim=True) + eps) * gain
+    return v, _shift_rows(u, mix, state, q_offsets, slot_ids).to(out_dtype)
+
+
+def _act(z, kind, params=(0.0, 0.0)):
+    if kind == "xielu":
+        neg = torch.clamp(z, max=0)
+        return torch.where(z > 0, params[0] * z * z + 0.5 * z, params[1] * (torch.expm1(neg) - neg) + 0.5 * z)
     if kind == "gelu_tanh":
         return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
     if kind == "relu_squared":
@@ -148,16 +185,16 @@ def _act(z, kind):
     raise ValueError(kind)
 
 
-def activation(x, kind):
-    x.copy_(_act(x.to(F64), kind).to(x.dtype))
+def activation(x, kind, params=(0.0, 0.0)):
+    x.copy_(_act(x.to(F64), kind, params).to(x.dtype))
     return x
 
 
-def gemm_act(x, w, kind, out_dtype):
-    return _act(x.to(F64) @ w.to(F64).T, kind).to(out_dtype)
+def gemm_act(x, w, kind, out_dtype, params=(0.0, 0.0)):
+    return _act(x.to(F64) @ w.to(F64).T, kind, params).to(out_dtype)
 
 
-def grouped_gemm(x, w, out, rows, gate=None, activation=None):
+def grouped_gemm(x, w, out, rows, gate=None, activation=None, gate_per_group=False):
     G, N, K = w.shape
     for g in range(G):
         xs = x.tensor[:rows, x.column + g * x.group: x.column + g * x.group + K].to(F64)
@@ -165,7 +202,8 @@ def grouped_gemm(x, w, out, rows, gate=None, activation=None):
         if activation:
             y = _act(y, activation)
         if gate is not None:
-            y = y * torch.sigmoid(gate.tensor[:rows, gate.column + g * gate.group: gate.column + g * gate.group + N].to(F64))
+            width = 1 if gate_per_group else N
+            y = y * torch.sigmoid(gate.tensor[:rows, gate.column + g * gate.group: gate.column + g * gate.group + width].to(F64))
         out.tensor[:rows, out.column + g * out.group: out.column + g * out.group + N] = y.to(out.tensor.dtype)
 
 
@@ -188,10 +226,14 @@ def _turn(part, cs, rd, pairing):
     return out
 
 
-def latent_prepare(proj, heads, dim, rot, rank, norm_weight, eps, positions, rope_table, pairing, cache, slots, qa):
+def latent_prepare(proj, heads, dim, rot, rank, norm_weight, eps, positions, rope_table, pairing, cache, slots, qa,
+                   q=None, kv_column=None):
     T = proj.shape[0]
-    q = proj[:, :heads * (dim + rot)].view(T, heads, dim + rot).to(F64)
-    down = proj[:, heads * (dim + rot): heads * (dim + rot) + rank + rot].to(F64)
+    if q is None:
+        q, kv_column = proj, heads * (dim + rot)
+    kv_column = int(kv_column or 0)
+    q = q[:, :heads * (dim + rot)].reshape(T, heads, dim + rot).to(F64)
+    down = proj[:, kv_column: kv_column + rank + rot].to(F64)
     c = down[:, :rank]
     c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * norm_weight.to(F64)
     cs = rope_table[positions.long()].to(F64) if rope_table is not None and rot else None
@@ -209,7 +251,7 @@ def latent_prepare(proj, heads, dim, rot, rank, norm_weight, eps, positions, rop
 
 
 def latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page_size, scale, window=0,
-                     plan=None, max_ctx=0):
+                     plan=None, max_ctx=0, sink=None):
     T = qa.shape[0]
     q = qa.view(T, heads, rank + rot).to(F64)
     out = torch.zeros(T, heads, rank, dtype=F64, device=qa.device)
@@ -223,7 +265,10 @@ def latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cach
         assert (pages >= 0).all(), "latent attention reads a page that was given back"
         offs = torch.tensor([j % page_size for j in js], dtype=torch.long)
         rows = cache[pages, offs].to(F64)                  # [n, rank + rot]
-        w = torch.softmax((q[t] @ rows.T) * scale, dim=-1)  # [heads, n]
+        s = (q[t] @ rows.T) * scale                         # [heads, n]
+        if sink is not None:                                # one more term in the denominator, no row
+            s = torch.cat([s, sink.to(F64)[:, None]], dim=-1)
+        w = torch.softmax(s, dim=-1)[:, :len(js)]
         out[t] = w @ rows[:, :rank]
     return out.reshape(T, heads * rank).to(qa.dtype)
 
@@ -240,6 +285,36 @@ def moe_route(logits, top, renormalise=True, eps=1e-20, large_tiles=False):
     r = _Routing()
     r.ids, r.weights = ids.to(torch.int32), picked.to(torch.float32)
     return r
+
+
+def moe_route_sigmoid(logits, top, correction=None, groups=1, keep=1, scale=1.0, large_tiles=False):
+    T, E = logits.shape
+    s = torch.sigmoid(logits.to(F64))
+    choice = s + correction.to(F64) if correction is not None else s.clone()
+    if groups > 1:
+        per = E // groups
+        ranks = torch.topk(choice.view(T, groups, per), min(2, per), dim=-1).values.sum(-1)
+        kept = torch.zeros(T, groups, dtype=torch.bool)
+        kept.scatter_(1, torch.topk(ranks, keep, dim=-1).indices, True)
+        choice = choice.masked_fill(~kept.repeat_interleave(per, dim=1), float("-inf"))
+    ids = torch.topk(choice, top, dim=-1).indices
+    r = _Routing()
+    r.ids, r.weights = ids.to(torch.int32), (torch.gather(s, 1, ids) * scale).to(torch.float32)
+    return r
+
+
+def lightning_prepare(proj, heads, key_dim, value_dim, decay):
+    T = proj.shape[0]
+    nk, nv = heads * key_dim, heads * value_dim
+
+    def silu(z):
+        return z * torch.sigmoid(z)
+    p = proj.to(F64)
+    coef = torch.zeros(5, T, nk, dtype=F64)
+    coef[0] = decay.to(F64).repeat_interleave(key_dim)[None, :]
+    coef[3] = silu(p[:, nk:2 * nk])
+    coef[4] = silu(p[:, :nk])
+    return coef.to(torch.float32), silu(p[:, 2 * nk:2 * nk + nv]).to(torch.float32)
 
 
 def moe_experts(x, w, routing, out_dtype, activation=None, gather=False):
@@ -461,7 +536,8 @@ ALL = ("layer_norm", "layer_norm_act", "embedding_sinusoid", "gated_activation",
        "check_delta_sizes", "general_delta_prepare", "gated_delta_prepare", "conv_tail_update", "delta_scan",
        "head_gate_norm", "moe_route_logits", "moe_combine_shared", "feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample", "dynamic_tanh", "stream_add", "activation", "gemm_act", "grouped_gemm",
-       "latent_prepare", "latent_attention", "moe_route", "moe_experts", "moe_combine")
+       "latent_prepare", "latent_attention", "moe_route", "moe_experts", "moe_combine",
+       "scale_", "token_shift", "rms_shift", "moe_route_sigmoid", "lightning_prepare")
 
 
 def install(monkeypatch):
