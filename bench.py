@@ -383,6 +383,31 @@ def larupel_design_config(name, routed=True):
             "initializer_range": 0.02, "layers": layers}
 
 
+def kikunex_design_config(name, routed=True):
+    """The Kikunex decoder at the same width, heads, head size, feed-forward width, vocabulary and
+    depth: lightning attention and latent attention in turn (heads of 128; the latent layers as
+    Pubodra's: 128 plain + 64 rotated query/key entries, values of 128, a latent of 512, window 4,096,
+    plus queries through a latent of 1,536); layers 1 and 2, one of each mixer, have routed
+    feed-forwards (4 of 32 experts of ff / 4, in 4 groups of which 2 are kept; ``routed`` False: dense
+    ones), the other two dense ones."""
+    width, heads, ff = DESIGN_SIZES[name]
+    lightning = {"heads": heads, "dim": 128, "vdim": 128,
+                 "decay": [1.0 - 2.0 ** (-5.0 - 5.0 * h / max(1, heads - 1)) for h in range(heads)]}
+    latent = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 1536,
+              "scale": 192 ** -0.5, "mask": {"size": 4096}, "rot": {"base": 1000000.0, "dims": 64}}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4},
+           "router": {"experts": 32, "top": 4, "groups": {"count": 4, "keep": 2}, "scale": 2.5}}
+    if not routed:
+        moe = dense
+    layers = [{"type": "lightning", "mixer": lightning, "mlp": dense},
+              {"type": "latent_attention", "mixer": latent, "mlp": moe},
+              {"type": "lightning", "mixer": lightning, "mlp": moe},
+              {"type": "latent_attention", "mixer": latent, "mlp": dense}]
+    return {"architecture": "Kikunex", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
+            "logit_scale": 0.5, "initializer_range": 0.02, "layers": layers}
+
+
 def design_run(cfg, dtype, dev, block_size, prompt, batches, context, steps):
     """Prompt and decode throughput of one configuration through the runner's own step."""
     import torch
@@ -465,10 +490,11 @@ def designs_workload(args, dev):
                 results[key] = design_run(pubodra, dtype, dev, args.block_size, args.prefill_tokens, batches,
                                           args.design_context, args.steps)
                 say(f"{key}: {results[key]}")
-        for model in ("larupel", "larupel_dense"):
+        for model in ("larupel", "larupel_dense", "kikunex", "kikunex_dense"):
             if model in wanted:
                 key = f"{name}/{model}"
-                results[key] = design_run(larupel_design_config(name, routed=model == "larupel"), dtype, dev,
+                make = larupel_design_config if model.startswith("larupel") else kikunex_design_config
+                results[key] = design_run(make(name, routed="dense" not in model), dtype, dev,
                                           args.block_size, args.prefill_tokens, batches, args.design_context, args.steps)
                 say(f"{key}: {results[key]}")
     head = f"decode_b{batches[0]}_ctx{args.design_context}"
@@ -518,7 +544,7 @@ def main() -> int:
     ap.add_argument("--design-sizes", default="w2048,w4096", help="designs: which of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-batches", default="8,64", help="designs: decode batch sizes")
     ap.add_argument("--design-models", default="qwen3,pubodra_dense,pubodra_routed,larupel",
-                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel, larupel_dense")
+                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel, larupel_dense, kikunex, kikunex_dense")
     ap.add_argument("--design-context", type=int, default=2048, help="designs: tokens a decoding request holds")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "designs"],
                     help="decode: the default line; mixed: only the 0.6B-shaped mixed workload, as a line of its own")
