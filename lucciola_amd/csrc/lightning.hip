@@ -34,9 +34,43 @@ __global__ void lightning_prepare_kernel(const float* __restrict__ proj, int col
     }
 }
 
+// One workgroup per token: all heads' read-outs together divided by their common root mean square, times
+// a weight, times sigmoid(gate); o, gates and the weight float32, the result in the activation type.
+template <typename T>
+__global__ void lightning_readout_kernel(const float* __restrict__ o, const float* __restrict__ gates, int gate_cols,
+                                         int gate_column, const float* __restrict__ weight, float eps, int n,
+                                         T* __restrict__ out) {
+    __shared__ float scratch[16];
+    const float* x = o + (size_t)blockIdx.x * n;
+    const float* g = gates + (size_t)blockIdx.x * gate_cols + gate_column;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(x[i], x[i], ss);
+    const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+    T* dst = out + (size_t)blockIdx.x * n;
+    for (int i = threadIdx.x; i < n; i += blockDim.x)
+        dst[i] = from_f32<T>(x[i] * inv * weight[i] / (1.f + expf(-g[i])));
+}
+
 }  // namespace lc
 
 using namespace lc;
+
+// o float32 [T, n]; gates float32 [T, gate_cols], the row's n gates from gate_column on; weight float32 [n]
+LC_API int lc_lightning_readout(const float* o, const float* gates, int gate_cols, int gate_column, const float* weight,
+                                float eps, int T, int n, void* out, int dt, hipStream_t stream) {
+    LC_CHECK(T >= 0 && n > 0 && gate_column >= 0 && gate_column + n <= gate_cols, "lightning readout: bad sizes");
+    if (T == 0) return 0;
+    LC_CHECK(o && gates && weight && out, "lightning readout: null pointer");
+    const int threads = n >= 2048 ? 512 : (n >= 512 ? 256 : (n >= 128 ? 128 : 64));
+    if (dt == DT_F32)
+        lightning_readout_kernel<float><<<T, threads, 0, stream>>>(o, gates, gate_cols, gate_column, weight, eps, n, (float*)out);
+    else if (dt == DT_BF16)
+        lightning_readout_kernel<bf16><<<T, threads, 0, stream>>>(o, gates, gate_cols, gate_column, weight, eps, n, (bf16*)out);
+    else
+        LC_CHECK(false, "lightning readout: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("lightning_readout");
+    return 0;
+}
 
 LC_API int lc_lightning_prepare(const float* proj, int cols, int T, int heads, int dk, int dv, const float* decay,
                                 float* coef, float* v_out, hipStream_t stream) {

@@ -122,7 +122,7 @@ __global__ void rms_shift_kernel(const float* __restrict__ h, const TD* __restri
         ss_other = fmaf(u, u, ss_other);
     }
     ss_own = block_sum(ss_own, scratch);
-    ss_other = block_sum(ss_other, scratch);
+    ss_other = other == t ? ss_own : block_sum(ss_other, scratch);      // a lone token: one row, one sum
     const float inv_own = g / sqrtf(ss_own / (float)n + eps), inv_other = g / sqrtf(ss_other / (float)n + eps);
     float* st = head ? state + (size_t)slot_ids[r] * n : nullptr;
     float* out_h = h_out + (size_t)t * n;

@@ -88,6 +88,7 @@ _SIGNATURES = {
     "lc_moe_route": "piiiifppp",
     "lc_moe_route_sigmoid": "ppiiiiifppp",
     "lc_lightning_prepare": "piiiiipppp",
+    "lc_lightning_readout": "ppiipfiipip",
     "lc_moe_lists": "piiiippppp",
     "lc_moe_combine": "pppiiipip",
     "lc_layer_norm": "ppippfpppfpiiiiip",
@@ -1734,3 +1735,21 @@ def lightning_prepare(proj: torch.Tensor, heads: int, key_dim: int, value_dim: i
         _call("lc_lightning_prepare", _ptr(proj), proj.shape[1], T, heads, key_dim, value_dim, _ptr(decay), _ptr(coef),
               _ptr(v), _stream())
     return coef, v
+
+
+def lightning_readout(o: torch.Tensor, gates: torch.Tensor, gate_column: int, weight: torch.Tensor, eps: float,
+                      out_dtype: torch.dtype) -> torch.Tensor:
+    """Every row of float32 ``o`` [T, n] (all heads side by side) divided by its root mean square (eps inside
+    the root), times ``weight`` [n], times sigmoid(g) with g the float32 columns ``gate_column`` .. + n of
+    ``gates``.  -> [T, n] of ``out_dtype``."""
+    _need(o, "lightning_readout o", torch.float32, 2)
+    _need(gates, "lightning_readout gates", torch.float32, 2)
+    _need(weight, "lightning_readout weight", torch.float32, 1)
+    T, n = o.shape
+    if gates.shape[0] != T or gate_column < 0 or gate_column + n > gates.shape[1] or weight.shape[0] != n:
+        raise KernelError("lightning_readout: the gates or the weight do not fit the rows")
+    out = torch.empty((T, n), dtype=out_dtype, device=o.device)
+    if T:
+        _call("lc_lightning_readout", _ptr(o), _ptr(gates), gates.shape[1], gate_column, _ptr(weight), float(eps), T, n,
+              _ptr(out), _dt(out), _stream())
+    return out

@@ -63,8 +63,7 @@ class Lightning(Part):
         coef, v = ops.lightning_prepare(proj, self.nh, self.dk, self.dv, self.decay)
         o = ops.delta_scan(coef, v, state, batch.q_offsets, batch.slot_ids, batch.num_requests,
                            self.nh, self.dk, self.dv)
-        # one norm over all heads together: a "head" of heads * value_dim entries
-        nv = self.nh * self.dv
-        y = ops.head_gate_norm(o, proj, 2 * self.nh * self.dk + nv, self.norm, True, self.norm_eps, "sigmoid",
-                               1, nv, self.dtype)
+        # one norm over all heads together, the weight and the gate in the same kernel
+        y = ops.lightning_readout(o, proj, 2 * self.nh * self.dk + self.nh * self.dv, self.norm, self.norm_eps,
+                                  self.dtype)
         return ops.gemm(y, self.o, self.dtype, defer=True)

@@ -317,6 +317,13 @@ def lightning_prepare(proj, heads, key_dim, value_dim, decay):
     return coef.to(torch.float32), silu(p[:, 2 * nk:2 * nk + nv]).to(torch.float32)
 
 
+def lightning_readout(o, gates, gate_column, weight, eps, out_dtype):
+    x = o.to(F64)
+    n = x.shape[1]
+    inv = torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    return (x * inv * weight.to(F64) * torch.sigmoid(gates[:, gate_column:gate_column + n].to(F64))).to(out_dtype)
+
+
 def moe_experts(x, w, routing, out_dtype, activation=None, gather=False):
     """Rows in (token, choice) order here: the order of the sorted rows is the kernels' own matter."""
     T, top = routing.ids.shape
@@ -537,7 +544,7 @@ ALL = ("layer_norm", "layer_norm_act", "embedding_sinusoid", "gated_activation",
        "head_gate_norm", "moe_route_logits", "moe_combine_shared", "feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample", "dynamic_tanh", "stream_add", "activation", "gemm_act", "grouped_gemm",
        "latent_prepare", "latent_attention", "moe_route", "moe_experts", "moe_combine",
-       "scale_", "token_shift", "rms_shift", "moe_route_sigmoid", "lightning_prepare")
+       "scale_", "token_shift", "rms_shift", "moe_route_sigmoid", "lightning_prepare", "lightning_readout")
 
 
 def install(monkeypatch):

@@ -1,0 +1,678 @@
+"""The Kikunex design on the GPU: every kernel it brought against the plain torch version of the same
+operation, and the engine against the plain whole-sequence implementation (``plain_kikunex``) in the
+four families of traces, in float32 and in bfloat16."""
+import pytest
+import torch
+
+import kikunex_configs as kc
+import plain_kikunex
+import reference_ops
+import traces
+from helpers import make_runner, prompts_for, random_weights, replay
+from lucciola_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+# A row's error: root mean square of the difference of the logits, means taken off, over that of the
+# plain logits.  In bfloat16 the roundings of the activations between the kernels put the median row of
+# these narrow, deep models at a few percent, and a router's choice between two experts whose scores
+# nearly tie can fall the other way, which changes that row by any amount: the bound is on the median
+# row, on the share of rows over 10 % and on the share of rows that are unrelated.  What a fault of the
+# cache, the state or the batch does wrong shows in many rows, and in float32.
+TOL = {"float32": 4e-5, "bfloat16": 1e-1}
+LENGTHS = {"A": [5, 1, 47, 90, 130], "B": [2, 61, 33, 100], "C": [150, 9, 230, 70]}
+_cache = {}
+
+
+def weights_for(cfg, seed, std=kc.STD):
+    """Random weights; the routers' four times as large, so that few choices are close calls; sinks and
+    shift rates of a size that shows when they are left out."""
+    weights = random_weights(dict(cfg, initializer_range=std), seed)
+    g = torch.Generator().manual_seed(seed)
+    for name in weights:
+        if name.endswith(".router"):
+            weights[name] = (weights[name].float() * 4).to(weights[name].dtype)
+        if name.endswith(".sink"):
+            weights[name] = (torch.randn(weights[name].shape, generator=g) * 1.5).to(weights[name].dtype)
+        if name.endswith(".shift"):
+            weights[name] = torch.rand(weights[name].shape, generator=g).to(weights[name].dtype)
+        if name.endswith(".correction"):
+            weights[name] = (torch.randn(weights[name].shape, generator=g) * 0.3).to(weights[name].dtype)
+    return weights
+
+
+def case(key):
+    if key not in _cache:
+        cfg, page, seed = kc.ALL[key]
+        weights = weights_for(cfg, seed)
+        prompts = prompts_for({"vocab_size": cfg["vocab"]}, LENGTHS[key], seed)
+        refs = {n: plain_kikunex.forward(cfg, weights, ids) for n, ids in prompts.items()}
+        _cache[key] = (cfg, page, weights, prompts, refs)
+    return _cache[key]
+
+
+def check_rows(got, prompts, refs, dtype, every=True):
+    errors = []
+    for name, ids in prompts.items():
+        for pos in range(len(ids)):
+            if (name, pos) not in got:
+                assert not every, f"{name} position {pos}: no logits"
+                continue
+            row, ref = got[(name, pos)], refs[name][pos]
+            assert torch.isfinite(row).all(), f"{name} position {pos}: logits are not finite"
+            diff = row - ref
+            err = float((diff - diff.mean()).pow(2).mean().sqrt() / (ref - ref.mean()).pow(2).mean().sqrt())
+            errors.append((err, name, pos))
+    tol = TOL[str(dtype).replace("torch.", "")]
+    over = sorted(e for e in errors if e[0] > tol)
+    worst = max(errors)
+    if tol == TOL["bfloat16"]:
+        median = sorted(errors)[len(errors) // 2]
+        assert median[0] <= 0.04, f"the median row's error is {median[0]:.3e}"
+        assert len(over) <= max(1, len(errors) // 10), f"{len(over)} of {len(errors)} rows over {tol:.1e}"
+        unrelated = [e for e in errors if e[0] > 0.6]
+        assert len(unrelated) <= max(1, len(errors) // 50), f"{len(unrelated)} of {len(errors)} rows are unrelated"
+        return worst[0]
+    assert worst[0] <= 3 * tol, f"request {worst[1]} position {worst[2]}: error {worst[0]:.3e} (bound {tol:.1e})"
+    assert len(over) <= max(1, len(errors) // 50), (
+        f"{len(over)} of {len(errors)} rows over {tol:.1e}; first: request {over[0][1]} position {over[0][2]} "
+        f"({over[0][0]:.3e})")
+    return worst[0]
+
+
+def close(got, want, dtype, what, scale=1.0):
+    tol = (4e-6 if dtype == torch.float32 else 1.2e-2) * scale
+    err = float((got.double() - want.double()).abs().max() / want.double().abs().max().clamp_min(1e-9))
+    assert err < tol, f"{what}: relative error {err:.3e}"
+
+
+def dev(*tensors):
+    return [t.to(DEV) if t is not None else None for t in tensors]
+
+
+def request_lists(lengths, slots):
+    q_offsets = torch.tensor([sum(lengths[:i]) for i in range(len(lengths) + 1)], dtype=torch.int32)
+    tok_req = torch.tensor([r for r, n in enumerate(lengths) for _ in range(n)], dtype=torch.int32)
+    return tok_req, q_offsets, torch.tensor(slots, dtype=torch.int32)
+
+
+# ------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,lengths", [(50, [5, 1, 12]), (192, [1, 1, 1, 1]), (1030, [40]), (2560, [2, 3])])
+def test_token_shift_alone_and_with_its_norm(dtype, n, lengths):
+    """Two steps in a row over the same slots: the second one's first rows are blended with what the
+    first left in the state."""
+    g = torch.Generator().manual_seed(n)
+    slots = [3, 0, 5, 1][:len(lengths)]
+    tok_req, q_offsets, slot_ids = request_lists(lengths, slots)
+    T = sum(lengths)
+    mix = torch.rand(n, generator=g)
+    states = [torch.randn(6, n, generator=g) for _ in range(2)]
+    pairs = [(reference_ops, [s.clone() for s in states], "cpu"), (ops, [s.to(DEV) for s in states], DEV)]
+    for step in range(2):
+        x = torch.randn(T, n, generator=g).to(dtype)
+        h = torch.randn(T, n, generator=g) * 3
+        delta = torch.randn(T, n, generator=g).to(dtype) if step else None
+        outs = []
+        for o, (plain_state, fused_state), where in pairs:
+            lists = [t.to(where) for t in (tok_req, q_offsets, slot_ids)]
+            y = o.token_shift(x.to(where), mix.to(where), plain_state, *lists)
+            h_new, z = o.rms_shift(h.to(where), delta.to(where) if step else None, 1.3, 1e-5, mix.to(where), fused_state,
+                                   *lists, dtype)
+            outs.append((y.cpu(), h_new.cpu(), z.cpu(), plain_state.cpu(), fused_state.cpu()))
+        for got, want, what in zip(outs[1], outs[0], ("shifted rows", "stream", "normed and shifted rows", "state",
+                                                      "state of the fused kernel")):
+            close(got, want, dtype if what.endswith("rows") else torch.float32, f"step {step}: {what}")
+        assert torch.equal(outs[1][3][[2, 4]], states[0][[2, 4]]), "a slot of no request was written"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_xielu_scale_and_stream_add(dtype):
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(11, 37, generator=g) * 3).to(dtype)
+    x[0, :4] = torch.tensor([0.0, -1e-4, 1e-4, -30.0]).to(dtype)
+    for params in ((0.8, 1.3), (0.0, 0.5), (2.5, 0.7)):
+        want = reference_ops.activation(x.clone(), "xielu", params)
+        close(ops.activation(x.to(DEV), "xielu", params).cpu(), want, dtype, f"xielu {params}")
+        direct = plain_kikunex.xielu(x, *[_inverse_softplus(params[0]), _inverse_softplus(params[1] - 0.5)]) if params[0] else None
+        if direct is not None:
+            close(want, direct, dtype, "xielu against its definition")
+    logits = torch.randn(5, 33, generator=g)
+    assert torch.equal(ops.scale_(logits.to(DEV), 0.3).cpu(), logits * 0.3)
+    h, delta, more, vec = (torch.randn(7, 33, generator=g), torch.randn(7, 33, generator=g).to(dtype),
+                           torch.randn(7, 33, generator=g), torch.randn(33, generator=g))
+    want = h.clone()
+    reference_ops.stream_add(want, delta, vec, more)
+    got = h.to(DEV)
+    ops.stream_add(got, delta.to(DEV), vec.to(DEV), more=more.to(DEV))
+    assert torch.allclose(got.cpu(), want, atol=2e-6)
+
+
+def _inverse_softplus(y):
+    import math
+    return math.log(math.expm1(y))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_of_some_columns(dtype):
+    g = torch.Generator().manual_seed(4)
+    x, w = torch.randn(9, 70, generator=g).to(dtype), torch.rand(23, generator=g) + 0.5
+    want = reference_ops.rmsnorm_act(x, w, 1e-5, column=11)
+    close(ops.rmsnorm_act(x.to(DEV), w.to(DEV), 1e-5, column=11).cpu(), want, dtype, "columns 11..34")
+    assert want.shape == (9, 23)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,G,N,K", [(1, 3, 21, 7), (16, 2, 64, 32), (77, 5, 18, 304), (300, 4, 48, 128)])
+def test_grouped_product_with_a_gate_per_group(dtype, rows, G, N, K):
+    g = torch.Generator().manual_seed(rows + G)
+    x = torch.randn(rows, G * K, generator=g).to(dtype)
+    w = torch.randn(G, N, K, generator=g).bfloat16()
+    gate = torch.randn(rows, 5 + G, generator=g).to(dtype)
+    out_ref, out_dev = torch.zeros(rows, G * N, dtype=dtype), torch.zeros(rows, G * N, dtype=dtype, device=DEV)
+    reference_ops.grouped_gemm(ops.Strided(x, 0, K), w, ops.Strided(out_ref, 0, N), rows, ops.Strided(gate, 5, 1),
+                               gate_per_group=True)
+    ops.grouped_gemm(ops.Strided(x.to(DEV), 0, K), w.to(DEV), ops.Strided(out_dev, 0, N), rows,
+                     ops.Strided(gate.to(DEV), 5, 1), gate_per_group=True)
+    close(out_dev.cpu(), out_ref, dtype, "grouped product with one gate a group", scale=max(1.0, K / 100))
+    by_hand = (x[:, K:2 * K].double() @ w[1].double().T) * torch.sigmoid(gate[:, 6].double())[:, None] if G > 1 else None
+    if by_hand is not None:
+        close(out_ref[:, N:2 * N], by_hand, dtype, "the plain version against the definition")
+
+
+@pytest.mark.parametrize("T,E,top,groups,keep", [(1, 4, 4, 1, 1), (9, 6, 2, 3, 2), (70, 12, 3, 4, 1), (300, 8, 4, 2, 1),
+                                                 (5, 130, 8, 10, 3), (33, 512, 6, 64, 5), (17, 7, 1, 7, 2), (4, 5, 5, 1, 1)])
+def test_sigmoid_routing_with_groups(T, E, top, groups, keep):
+    g = torch.Generator().manual_seed(T + E)
+    logits = torch.randn(T, E, generator=g) * 2
+    correction = torch.randn(E, generator=g) * 0.5
+    want = reference_ops.moe_route_sigmoid(logits, top, correction, groups, keep, 1.7)
+    r = ops.moe_route_sigmoid(*dev(logits), top, correction.to(DEV), groups, keep, 1.7)
+    assert torch.equal(r.ids.cpu(), want.ids), "chosen experts"
+    assert torch.allclose(r.weights.cpu(), want.weights, atol=1e-6)
+    chosen, weights = plain_kikunex.route(logits, correction, {"top": top, "groups": {"count": groups, "keep": keep}, "scale": 1.7})
+    assert torch.equal(chosen.to(torch.int32), want.ids) and torch.allclose(weights.float(), want.weights, atol=1e-6)
+    starts = r.row_start.cpu().tolist()
+    assert starts[0] == 0 and starts[-1] == T * top and starts == sorted(starts)
+    none = ops.moe_route_sigmoid(*dev(logits), top, None, 1, 1, 1.0)
+    assert torch.equal(none.ids.cpu(), torch.topk(torch.sigmoid(logits.double()), top, dim=-1).indices.to(torch.int32))
+
+
+def test_a_negative_choice_score_inside_a_kept_group_wins():
+    logits = torch.tensor([[4.0, -9.0, -9.0, 0.5, 0.0, -3.0]])
+    correction = torch.tensor([0.0, 0.0, 0.0, 0.6, 0.6, -2.0])
+    r = ops.moe_route_sigmoid(logits.to(DEV), 3, correction.to(DEV), 2, 1, 2.0)
+    assert r.ids.cpu().tolist() == [[3, 4, 5]]
+    assert torch.allclose(r.weights.cpu()[0], torch.sigmoid(torch.tensor([0.5, 0.0, -3.0])) * 2.0, atol=1e-6)
+
+
+@pytest.mark.parametrize("heads,dk,dv,lengths", [(2, 16, 16, [5, 1, 40]), (3, 7, 9, [1, 1, 1, 1]), (2, 32, 64, [70]),
+                                                 (1, 128, 128, [33, 2]), (4, 48, 40, [9])])
+def test_lightning_kernels_against_the_recurrence(heads, dk, dv, lengths):
+    """Projections -> scan inputs -> scan -> gated read-out over two steps, against the token-by-token
+    recurrence written out."""
+    g = torch.Generator().manual_seed(heads * dk)
+    decay = torch.tensor([0.5, 0.9, 0.99, 1.0][:heads])
+    slots = [2, 0, 3, 1][:len(lengths)]
+    tok_req, q_offsets, slot_ids = request_lists(lengths, slots)
+    T, nk, nv = sum(lengths), heads * dk, heads * dv
+    state = torch.zeros(4, heads, dv, dk, device=DEV)
+    by_hand = torch.zeros(4, heads, dk, dv, dtype=torch.float64)
+    weight = torch.rand(nv, generator=g) + 0.5
+    for step in range(2):
+        proj = torch.randn(T, 2 * nk + 2 * nv + 3, generator=g)
+        coef, v = ops.lightning_prepare(proj.to(DEV), heads, dk, dv, decay.to(DEV))
+        c_ref, v_ref = reference_ops.lightning_prepare(proj, heads, dk, dv, decay)
+        close(coef.cpu(), c_ref, torch.float32, "scan inputs")
+        close(v.cpu(), v_ref, torch.float32, "values")
+        o = ops.delta_scan(coef, v, state, *dev(q_offsets, slot_ids), len(lengths), heads, dk, dv)
+        q = plain_kikunex.silu(proj[:, :nk]).view(T, heads, dk)
+        k = plain_kikunex.silu(proj[:, nk:2 * nk]).view(T, heads, dk)
+        val = plain_kikunex.silu(proj[:, 2 * nk:2 * nk + nv]).view(T, heads, dv)
+        want = torch.zeros(T, heads, dv, dtype=torch.float64)
+        for r, slot in enumerate(slots):
+            for t in range(int(q_offsets[r]), int(q_offsets[r + 1])):
+                for h in range(heads):
+                    by_hand[slot, h] = float(decay[h]) * by_hand[slot, h] + torch.outer(k[t, h], val[t, h])
+                    want[t, h] = by_hand[slot, h].T @ q[t, h]
+        close(o.cpu(), want.view(T, nv), torch.float32, f"step {step}: read-outs", scale=10)
+        close(state.cpu().transpose(2, 3), by_hand, torch.float32, f"step {step}: states", scale=10)
+        for dtype in (torch.float32, torch.bfloat16):
+            y = ops.lightning_readout(o, proj.to(DEV), 2 * nk + nv, weight.to(DEV), 1e-5, dtype)
+            w64 = want.view(T, nv)
+            ref = plain_kikunex.unit_rms(w64, 1e-5) * weight.double() * torch.sigmoid(proj[:, 2 * nk + nv:2 * nk + 2 * nv].double())
+            close(y.cpu(), ref, dtype, "gated read-out", scale=10)
+
+
+def test_a_far_write_is_read_back_by_lightning_attention():
+    """A pair written at the sequence's first token under a key that no later token uses is read back 600
+    tokens later at decay^599: at full strength where the head never forgets."""
+    heads, dk, dv, T = 2, 16, 16, 600
+    decay = torch.tensor([1.0, 0.995])
+    big, small = 20.0, -40.0                 # silu(20) = 20 (1 - 2e-9), silu(-40) = -2e-16
+    proj = torch.full((T, heads * (2 * dk + dv)), small)
+    for h in range(heads):
+        proj[0, heads * dk + h * dk] = big                     # the first token's key: channel 0
+        proj[1:, heads * dk + h * dk + 1] = big                # every other token's: channel 1
+        proj[T - 1, h * dk] = big                              # the last token reads channel 0
+    v_cols = slice(2 * heads * dk, 2 * heads * dk + heads * dv)
+    proj[:, v_cols] = torch.randn(T, heads * dv, generator=torch.Generator().manual_seed(3)) * 2
+    coef, v = ops.lightning_prepare(proj.to(DEV), heads, dk, dv, decay.to(DEV))
+    state = torch.zeros(1, heads, dv, dk, device=DEV)
+    tok_req, q_offsets, slot_ids = request_lists([T], [0])
+    o = ops.delta_scan(coef, v, state, *dev(q_offsets, slot_ids), 1, heads, dk, dv).cpu().view(T, heads, dv)
+    first = plain_kikunex.silu(proj[0, v_cols]).view(heads, dv)
+    for h in range(heads):
+        close(o[T - 1, h], first[h] * (big * 0.9999999979) ** 2 * float(decay[h]) ** (T - 1), torch.float32, f"decay {float(decay[h])}", scale=30)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,dim,rot,rank,page,window", [(3, 7, 10, 21, 8, 17), (4, 16, 8, 32, 4, 0), (5, 0, 12, 40, 16, 70),
+                                                            (9, 8, 16, 304, 16, 130), (2, 32, 16, 64, 16, 40)])
+def test_latent_kernels_with_queries_of_their_own_and_sinks(dtype, heads, dim, rot, rank, page, window):
+    """Two requests of unequal length written to scattered pages in two portions each, then read; the
+    queries come from a tensor of their own, every head has a sink."""
+    g = torch.Generator().manual_seed(heads * 100 + rank)
+    lengths = [150, 37]
+    pages = sum(-(-n // page) for n in lengths) + 3
+    kv_column = 5
+    caches = [torch.zeros(pages, page, rank + rot, dtype=dtype), torch.zeros(pages, page, rank + rot, dtype=dtype, device=DEV)]
+    table = torch.randn(200, rot, generator=g)
+    w = torch.rand(rank, generator=g) + 0.5
+    sink = torch.randn(heads, generator=g) * 2
+    order = torch.randperm(pages, generator=g).tolist()
+    per = -(-max(lengths) // page)
+    block_table = torch.full((2, per), -1, dtype=torch.int32)
+    for r, n in enumerate(lengths):
+        for b in range(-(-n // page)):
+            block_table[r, b] = order.pop()
+    done = [0, 0]
+    for cut in (0.6, 1.0):
+        tok_req, positions = [], []
+        for r, n in enumerate(lengths):
+            upto = int(n * cut)
+            tok_req += [r] * (upto - done[r])
+            positions += list(range(done[r], upto))
+            done[r] = upto
+        T = len(tok_req)
+        tok_req, positions = torch.tensor(tok_req, dtype=torch.int32), torch.tensor(positions, dtype=torch.int32)
+        slots = (block_table[tok_req.long(), (positions // page).long()] * page + positions % page).to(torch.int32)
+        proj = torch.randn(T, kv_column + rank + rot + 2, generator=g).to(dtype)
+        q = torch.randn(T, heads * (dim + rot), generator=g).to(dtype)
+        latent_q = torch.randn(T, heads, rank, generator=g).to(dtype)
+        outs = []
+        for where, cache in zip(("cpu", DEV), caches):
+            o = reference_ops if where == "cpu" else ops
+            qa = torch.zeros(T, heads * (rank + rot), dtype=dtype, device=where)
+            o.latent_prepare(proj.to(where), heads, dim, rot, rank, w.to(where), 1e-5, positions.to(where),
+                             table.to(where), "half", cache, slots.to(where), qa, q=q.to(where), kv_column=kv_column)
+            qa.view(T, heads, rank + rot)[..., :rank] = latent_q.to(where)
+            outs.append((qa.cpu(), o.latent_attention(qa, heads, rank, rot, tok_req.to(where), positions.to(where),
+                                                      block_table.to(where), cache, page, 0.3, window,
+                                                      sink=sink.to(where)).cpu()))
+        close(outs[1][0], outs[0][0], dtype, "rotated queries")
+        close(caches[1].cpu(), caches[0], dtype, "cache rows")
+        caches[1].copy_(caches[0])
+        close(outs[1][1], outs[0][1], dtype, "latent attention with sinks", scale=max(1.0, (rank + rot) / 300) ** 0.5)
+
+
+@pytest.mark.parametrize("heads,rank,rot,page,window", [(4, 32, 16, 16, 0), (3, 48, 8, 4, 37), (16, 64, 32, 16, 100),
+                                                        (70, 16, 0, 8, 0), (9, 512, 64, 16, 130)])
+def test_sinks_on_the_matrix_cores(heads, rank, rot, page, window):
+    """A step of portions beside lone tokens, then lone tokens alone, with a sink per head (one of them
+    far above every score, one far below): the matrix-core kernel, also with the keys of a tile shared
+    out over workgroups, against the plain version."""
+    from lucciola_amd.engine.batch import HostLayout, Plan
+    g = torch.Generator().manual_seed(heads + rank)
+    sink = torch.randn(heads, generator=g) * 2
+    sink[0] = 30.0
+    sink[-1] = -30.0
+    for history, fresh in (([150, 0, 299, 33, 64], [40, 2, 1, 17, 1]), ([299, 0, 64, 31, 700], [1, 1, 1, 1, 1])):
+        n_pages = sum(-(-(h + f) // page) for h, f in zip(history, fresh)) + 2
+        order = torch.randperm(n_pages, generator=g).tolist()
+        width = max(-(-(h + f) // page) for h, f in zip(history, fresh))
+        block_table = torch.full((len(history), width), -1, dtype=torch.int32)
+        cache = (torch.randn(n_pages, page, rank + rot, generator=g) * 0.5).bfloat16()
+        for r, (h, f) in enumerate(zip(history, fresh)):
+            for b in range(-(-(h + f) // page)):
+                block_table[r, b] = order.pop()
+        q_start = [0]
+        for f in fresh:
+            q_start.append(q_start[-1] + f)
+        T = q_start[-1]
+        tok_req = torch.tensor([r for r, f in enumerate(fresh) for _ in range(f)], dtype=torch.int32)
+        positions = torch.tensor([history[r] + i for r, f in enumerate(fresh) for i in range(f)], dtype=torch.int32)
+        qa = torch.randn(T, heads * (rank + rot), generator=g).bfloat16()
+        arrays, info = ops.plan_latent_attention(HostLayout(len(fresh), T, q_start, history, page, max(fresh) == 1))
+        plan = Plan({k: torch.from_numpy(v).to(DEV) for k, v in arrays.items()}, info)
+        want = reference_ops.latent_attention(qa, heads, rank, rot, tok_req, positions, block_table, cache, page, 0.2,
+                                              window, sink=sink)
+        args = (qa.to(DEV), heads, rank, rot, tok_req.to(DEV), positions.to(DEV), block_table.to(DEV), cache.to(DEV),
+                page, 0.2, window)
+        close(ops.latent_attention(*args, sink=sink.to(DEV)).cpu(), want, torch.bfloat16, "general kernel")
+        close(ops.latent_attention(*args, plan=plan, max_ctx=701, sink=sink.to(DEV)).cpu(), want, torch.bfloat16,
+              "matrix-core kernel")
+        close(ops.latent_attention(*args, plan=plan, max_ctx=1 << 20, sink=sink.to(DEV)).cpu(), want, torch.bfloat16,
+              "matrix-core kernel with shares")
+        assert float(want.view(T, heads, rank)[:, 0].abs().max()) < 1e-3, "a sink of 30 leaves the keys no weight"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window,page", [(33, 16), (64, 16), (17, 4), (0, 8)])
+def test_one_key_carries_the_weight_beside_a_sink(dtype, window, page):
+    """Among 300 cached rows one row's score stands out; it is put far back, on both sides of every page
+    border near the window's edge, just inside and just outside the window, and is read by a lone token
+    and by the last row of a portion.  Where the query sees it the result is that row's latent, whatever
+    the sinks; where it does not, it is not."""
+    heads, rank, rot, n = 2, 16, 4, 300
+    g = torch.Generator().manual_seed(window + page)
+    pages = -(-n // page) + 2
+    order = torch.randperm(pages, generator=g).tolist()
+    block_table = torch.tensor([order[:-(-n // page)]], dtype=torch.int32)
+    base = (torch.randn(n, rank + rot, generator=g) * 0.1)
+    marker = torch.zeros(rank + rot)
+    marker[3] = 6.0
+    p = n - 1
+    edge = p - window + 1 if window else 0
+    sink = torch.tensor([2.0, 5.0])
+    places = sorted({0, 1, edge - 1, edge, edge + 1, p - 1, p} | {b + d for b in range(edge - page, edge + page + 1, 1)
+                                                                  if b % page == 0 for d in (-1, 0)})
+    for place in [j for j in places if 0 <= j <= p]:
+        rows = base.clone()
+        rows[place] = marker
+        cache = torch.zeros(pages, page, rank + rot, dtype=dtype)
+        for j in range(n):
+            cache[block_table[0, j // page], j % page] = rows[j].to(dtype)
+        qa = torch.zeros(heads * (rank + rot))
+        qa[3] = qa[rank + rot + 3] = 4.0
+        seen = place >= edge
+        for portion in (1, 7):
+            T = portion
+            positions = torch.arange(p - T + 1, p + 1, dtype=torch.int32)
+            q = qa.to(dtype).repeat(T, 1)
+            args = (heads, rank, rot, torch.zeros(T, dtype=torch.int32), positions, block_table)
+            want = reference_ops.latent_attention(q, *args, cache, page, 1.0, window, sink=sink)
+            got = ops.latent_attention(q.to(DEV), heads, rank, rot, args[3].to(DEV), positions.to(DEV),
+                                       block_table.to(DEV), cache.to(DEV), page, 1.0, window, sink=sink.to(DEV)).cpu()
+            close(got, want, dtype, f"marker at {place}, window {window}, portion of {portion}")
+            last = got[-1].float().view(heads, rank)
+            assert (float(last[0, 3]) > 5.5) == seen, f"marker at {place} (edge {edge}): seen is {seen}"
+
+
+# ------------------------------------------------------------------ the engine
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+@pytest.mark.parametrize("family", ["whole", "tail", "chunked", "mixed"])
+def test_replay_families(dtype, key, family):
+    cfg, page, weights, prompts, refs = case(key)
+    steps = {"whole": traces.whole, "tail": traces.tail_decode, "chunked": traces.chunked,
+             "mixed": traces.mixed}[family](prompts)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    got = replay(runner, steps)
+    assert len(got) == sum(len(p) for p in prompts.values())
+    worst = check_rows(got, prompts, refs, dtype)
+    print(f"{key} {family} {dtype}: worst error {worst:.3e}")
+    assert not runner.cache.requests
+    for g in runner.cache.groups:
+        assert g.pool.num_free() == blocks
+
+
+def _one_layer(mixer, mlp, **more):
+    cfg = {"architecture": "Kikunex", "vocab": 97, "width": 40, "norm": {"eps": 2e-6}, "layers": [kc.layer(mixer, mlp)]}
+    cfg.update(more)
+    return cfg
+
+
+MECHANISMS = {
+    "attention alone": _one_layer(kc.latent(3, 8, 6, 5, 12, 9, 0.3, 11, base=200.0), None),
+    "attention, one head, no window": _one_layer(kc.latent(1, 9, 2, 7, 10, 40, 0.4, None), None, logit_scale=0.2),
+    "attention, everything rotated": _one_layer(kc.latent(2, 0, 12, 6, 8, 8, 0.3, 5, base=50.0), None),
+    "lightning alone": _one_layer(kc.lightning(3, 8, 5, (0.9, 1.0, 0.3)), None),
+    "lightning, one head of one channel": _one_layer(kc.lightning(1, 1, 1, (0.95,)), None, logit_scale=3.0),
+    "dense feed-forward": _one_layer(kc.lightning(2, 4, 4, (0.9, 0.8)), kc.dense(33)),
+    "every expert chosen": _one_layer(kc.latent(2, 4, 4, 4, 8, 8, 0.5, 64), kc.moe(12, 4, 4, scale=0.4)),
+    "one expert of many, groups of one": _one_layer(kc.lightning(2, 4, 4, (0.9, 0.8)), kc.moe(20, 70, 1, groups=70, keep=9, scale=3.0)),
+    "all groups kept": _one_layer(kc.latent(2, 4, 4, 4, 8, 8, 0.5, 64), kc.moe(16, 6, 3, groups=2, keep=2)),
+    "a stack run once": _one_layer(kc.lightning(2, 4, 4, (0.9, 0.8)), kc.dense(16), loop={"start": 0, "stop": 1, "times": 1}),
+    "one layer run four times": _one_layer(kc.latent(2, 4, 4, 4, 8, 8, 0.5, 7), kc.moe(16, 4, 2, groups=2, keep=1, scale=2.0),
+                                           loop={"start": 0, "stop": 1, "times": 4}),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(MECHANISMS))
+def test_each_mechanism(name, dtype):
+    """Models of one layer that have one mechanism each, with sizes of 1, of 0 and equal to one another,
+    fed whole, in portions and token by token."""
+    cfg = MECHANISMS[name]
+    weights = weights_for(cfg, 5, std=0.15 if dtype == "float32" else 0.06)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [23, 2, 58], 3)
+    refs = {n: plain_kikunex.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    every_token = [([(n, [t], [0])], [n] if i == len(ids) - 1 else []) for n, ids in prompts.items()
+                   for i, t in enumerate(ids)]
+    for steps in (traces.whole(prompts), traces.chunked(prompts, sizes=(2, 9, 3, 2, 17)), every_token):
+        runner = make_runner(cfg, weights, 4, 40, dtype, DEV)
+        check_rows(replay(runner, steps), prompts, refs, dtype)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_the_shift_in_one_kernel_and_in_two(fused):
+    cfg, page, weights, prompts, refs = case("B")
+    steps = traces.mixed(prompts)
+    runner = make_runner(cfg, weights, page, traces.max_live_tokens(steps, page) // page, "float32", DEV)
+    for layer in runner.model.layers:
+        layer.mixer_shift.fused = fused
+    check_rows(replay(runner, steps), prompts, refs, "float32")
+
+
+def test_the_first_tokens_and_a_shift_that_takes_the_whole_previous_row():
+    """With a shift rate of 1 a mixer reads only the previous token's row, and zeros at the first token;
+    prompts of one, two and three tokens, cut after every token."""
+    cfg, page, seed = kc.ALL["B"]
+    weights = weights_for(cfg, seed)
+    for name in weights:
+        if name.endswith(".shift"):
+            weights[name] = torch.ones_like(weights[name])
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [1, 2, 3, 19], seed)
+    refs = {n: plain_kikunex.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    for steps in (traces.whole(prompts), traces.chunked(prompts, sizes=(1, 1, 2, 3)), traces.mixed(prompts, decode_tail=2)):
+        runner = make_runner(cfg, weights, page, 16, "float32", DEV)
+        check_rows(replay(runner, steps), prompts, refs, "float32")
+
+
+def engine_for(cfg, weights, page, blocks, dtype, **kw):
+    from lucciola_amd.config.engine_config import EngineConfig
+    from lucciola_amd.config.registry import architecture_for
+    from lucciola_amd.engine.llm_engine import LLMEngine
+    from lucciola_amd.engine.loading import _build
+    from lucciola_amd.weights.loader import DictSource
+    arch = architecture_for(cfg)
+    config = arch.read_config(cfg)
+    model = _build(arch.model_spec(config), DictSource(weights), dtype, DEV)
+    return LLMEngine(model, config, EngineConfig(dtype=dtype, block_size=page, max_blocks=blocks, device=DEV, **kw))
+
+
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_greedy_generation_through_the_engine(key):
+    from lucciola_amd.sampling.sampler import SamplingParams
+    cfg, page, seed = kc.ALL[key]
+    weights = weights_for(cfg, seed, std=0.2)
+    prompts = list(prompts_for({"vocab_size": cfg["vocab"]}, [5, 11, 37], seed + 30).values())
+    engine = engine_for(cfg, weights, page, 64, "float32", max_tokens_per_step=16, max_seqs=4)
+    got = engine.generate(prompts, SamplingParams(max_new_tokens=8))
+    assert got == [plain_kikunex.greedy(cfg, weights, p, 8) for p in prompts]
+    engine.runner.cache.check()
+    assert not engine.runner.cache.requests
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_generation_survives_preemption(ahead):
+    """With so few pages that running requests are preempted and fed again from their start (into a
+    cleared slot), every request's tokens are the plain implementation's."""
+    from lucciola_amd.sampling.sampler import SamplingParams
+    cfg, page, seed = kc.ALL["B"]
+    weights = weights_for(cfg, seed, std=0.2)
+    prompts = list(prompts_for({"vocab_size": cfg["vocab"]}, [9, 14, 6, 11], seed + 40).values())
+    tight = engine_for(cfg, weights, page, 9, "float32", max_tokens_per_step=12, max_seqs=4, run_ahead=ahead)
+    got = tight.generate(prompts, SamplingParams(max_new_tokens=20))
+    assert tight.scheduler.num_preemptions > 0
+    for prompt, tokens in zip(prompts, got):
+        assert tokens == plain_kikunex.greedy(cfg, weights, prompt, 20)
+    tight.runner.cache.check()
+    assert not tight.runner.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "C"])
+def test_long_decoding_stale_pages_and_used_slots(dtype, key):
+    """A short prompt, then 260 tokens one by one (in bfloat16 through captured steps), past every
+    window, in a cache whose pages and slots hold other requests' rows and states when they are taken."""
+    cfg, page, seed = kc.ALL[key]
+    weights = weights_for(cfg, seed)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [268, 270], seed + 7)
+    refs = {n: plain_kikunex.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = traces.tail_decode(prompts, tail=260)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV, max_seqs=1)
+    for stored in runner.cache.storage.values():
+        for need in stored:
+            for t in (need if isinstance(need, (tuple, list)) else (need,)):
+                t.normal_(0, 30.0)
+    check_rows(replay(runner, steps), prompts, refs, dtype)
+    if dtype == "bfloat16":
+        assert runner.graph_replays > 200
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from lucciola_amd.weights.random_init import write_model_folder
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = kc.ALL["B"]
+    folder = write_model_folder(str(tmp_path / "model"), dict(cfg, initializer_range=kc.STD), seed)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [70, 33, 50, 3, 61], seed)
+    steps = traces.mixed(prompts, seed=3)
+    lines, index, fed = [], {}, {}
+    for i, (entries, end) in enumerate(steps):
+        lines.append(json.dumps({"step": i, "end": end, "entries": [{"id": n, "tokens": t, "want": w} for n, t, w in entries]}))
+        rows = []
+        for n, t, w in entries:
+            rows += [(n, fed.get(n, 0) + k) for k in w]
+            fed[n] = fed.get(n, 0) + len(t)
+        index[i] = rows
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(traces.max_live_tokens(steps, 64))],
+                          input="\n".join(lines) + "\n", text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [x for i in range(len(steps)) for x in ("done", str(i))]
+    got = {}
+    for i, rows in index.items():
+        data = np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"])
+        for r, key in enumerate(rows):
+            got[key] = torch.from_numpy(data[r].astype("float64"))
+    refs = {n: plain_kikunex.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    check_rows(got, prompts, refs, dtype)
+
+
+def test_float32_logits_do_not_depend_on_the_cut():
+    """The same bits whole, in portions and token by token: every sum's order follows from the token
+    alone."""
+    cfg, page, seed = kc.ALL["B"]
+    weights = weights_for(cfg, seed)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [75, 40], seed)
+    runs = []
+    for steps in (traces.whole(prompts), traces.chunked(prompts), traces.tail_decode(prompts, tail=30), traces.mixed(prompts)):
+        runs.append(replay(make_runner(cfg, weights, page, 40, "float32", DEV), steps))
+    for other in runs[1:]:
+        for key, row in runs[0].items():
+            assert torch.equal(row, other[key]), f"{key}: the bits differ between two cuts"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("key", ["A", "B", "C"])
+def test_a_batch_of_unequal_requests_against_each_alone(key, dtype):
+    """Four requests of unequal length in one step, then steps of lone tokens: every row against the same
+    request run alone (the same bits in float32; within rounding in bfloat16, where other rows in a step
+    mean other product kernels)."""
+    cfg, page, weights, prompts, refs = case(key)
+    names = list(prompts)[:4]
+    alone = {}
+    for n in names:
+        runner = make_runner(cfg, weights, page, 64, dtype, DEV)
+        alone.update(replay(runner, traces.whole({n: prompts[n]})))
+    runner = make_runner(cfg, weights, page, 64, dtype, DEV)
+    cut = {n: max(1, len(prompts[n]) - 3) for n in names}
+    steps = [([(n, prompts[n][:cut[n]], list(range(cut[n]))) for n in names], [])]
+    rest = {n: prompts[n][cut[n]:] for n in names}
+    longest = max(len(r) for r in rest.values())
+    for k in range(longest):
+        entries = [(n, [rest[n][k]], [0]) for n in names if k < len(rest[n])]
+        steps.append((entries, [n for n in names if k == len(rest[n]) - 1]))
+    steps[0] = (steps[0][0], [n for n in names if not rest[n]])
+    together = replay(runner, [s for s in steps if s[0]])
+    assert sorted(together) == sorted(alone)
+    errors = []
+    for row_key, row in alone.items():
+        if dtype == "float32":
+            assert torch.equal(row, together[row_key]), f"{row_key}: the bits differ between alone and in a batch"
+        else:
+            diff = row - together[row_key]
+            errors.append(float((diff - diff.mean()).pow(2).mean().sqrt() / (row - row.mean()).pow(2).mean().sqrt()))
+    if errors:      # a router's close call may fall the other way in a few rows
+        errors.sort()
+        assert errors[len(errors) // 2] < 0.03, f"median difference {errors[len(errors) // 2]:.3e}"
+        assert sum(e > 0.1 for e in errors) <= len(errors) // 10
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(14))
+def test_random_configurations(seed, dtype):
+    """Configurations drawn at random, requests in mixed steps with so few pages and slots that they are
+    used again, against the plain implementation."""
+    cfg, page = kc.random_configuration(seed)
+    weights = weights_for(cfg, 100 + seed)
+    prompts = prompts_for({"vocab_size": cfg["vocab"]}, [3, 120, 41, 77, 1, 150], seed)
+    refs = {n: plain_kikunex.forward(cfg, weights, ids) for n, ids in prompts.items()}
+    steps = traces.mixed(prompts, seed=seed)
+    blocks = traces.max_live_tokens(steps, page) // page
+    runner = make_runner(cfg, weights, page, blocks, dtype, DEV)
+    check_rows(replay(runner, steps), prompts, refs, dtype)
+    assert not runner.cache.requests
+
+
+def test_command_line(tmp_path):
+    """A model folder made from a configuration and a seed, then greedy tokens through
+    ``python -m lucciola_amd``: the architecture is found by config.json alone."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from lucciola_amd.weights.safetensors_io import SafetensorsFile
+    cfg, page, seed = kc.ALL["A"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(dict(cfg, initializer_range=0.2)))
+    folder = str(tmp_path / "model")
+    run = [sys.executable, "-m", "lucciola_amd"]
+    made = subprocess.run(run + ["--random-config", str(config_file), "--seed", "4", "--write-model", folder],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert made.returncode == 0, made.stderr[-2000:]
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        weights = {n: f.get(n).clone() for n in f.names()}
+    prompts = [[3, 17, 150, 9], [88] * 30 + [5, 6]]
+    proc = subprocess.run(run + ["--model", folder, "--dtype", "float32", "--max-new-tokens", "6", "--max-blocks", "64",
+                                 "--block-size", str(page), "--max-tokens-per-step", "12"]
+                          + [x for p in prompts for x in ("--prompt-ids", ",".join(map(str, p)))],
+                          cwd=root, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [[int(t) for t in line.split()] for line in proc.stdout.strip().splitlines()]
+    assert got == [plain_kikunex.greedy(cfg, weights, p, 6) for p in prompts]
