@@ -220,19 +220,27 @@ __device__ __forceinline__ void lds_rows(float (&dst)[ROWS], const float* generi
     }
 }
 
-// What a lane needs of one token: its run of each of the five vectors, and its column's value.
-template <int ROWS>
+// What a lane needs of one token: its run of each of the vectors, and its column's value.  REMOVE: the
+// recurrence has a removal term (five vectors: decay, probe, removal, write, read); else three (decay,
+// write, read), and probe and removal are never touched.
+template <int ROWS, bool REMOVE>
 struct TokenRows {
-    float decay[ROWS], probe[ROWS], removal[ROWS], write[ROWS], read_by[ROWS], value;
-    // stage: the stage's vectors [5][CHUNK][DKP] (`plane` floats a vector, `dkp` a token), values: [CHUNK][columns]
+    float decay[ROWS], probe[REMOVE ? ROWS : 1], removal[REMOVE ? ROWS : 1], write[ROWS], read_by[ROWS], value;
+    // stage: the stage's vectors [5 or 3][CHUNK][DKP] (`plane` floats a vector, `dkp` a token), values: [CHUNK][columns]
     __device__ __forceinline__ void load(const float* stage, const float* values, int tt, int lane, int col, int plane,
                                          int dkp, int columns) {
         const float* at = stage + tt * dkp + lane * ROWS;
-        lds_rows<ROWS>(probe, at + plane);
-        lds_rows<ROWS>(decay, at);
-        lds_rows<ROWS>(removal, at + 2 * plane);
-        lds_rows<ROWS>(write, at + 3 * plane);
-        lds_rows<ROWS>(read_by, at + 4 * plane);
+        if constexpr (REMOVE) {
+            lds_rows<ROWS>(probe, at + plane);
+            lds_rows<ROWS>(decay, at);
+            lds_rows<ROWS>(removal, at + 2 * plane);
+            lds_rows<ROWS>(write, at + 3 * plane);
+            lds_rows<ROWS>(read_by, at + 4 * plane);
+        } else {
+            lds_rows<ROWS>(decay, at);
+            lds_rows<ROWS>(write, at + plane);
+            lds_rows<ROWS>(read_by, at + 2 * plane);
+        }
         value = ((lds_cf*)values)[tt * columns + col];
     }
 };
@@ -247,19 +255,23 @@ struct TokenRows {
 // 594 for a 2,048-token request of 16 heads of 128 x 128.)
 // DEEP: a token's vectors are read a token ahead (more registers, fewer waves a SIMD: for steps
 // of long portions; steps of lone tokens are bound by the states' trip to memory and want the waves).
-template <int ROWS, int CHUNK, bool DEEP, int COLS>
+// REMOVE = false is the recurrence without its removal term, S <- diag(decay) S + write v^T, over three
+// vectors a token: then only the state's own multiply-add ties a token to the next (no sum over the
+// lanes stands before it), and the read-outs' sums of neighbouring tokens overlap.
+template <int ROWS, int CHUNK, bool DEEP, int COLS, bool REMOVE>
 __global__ __launch_bounds__(COLS * SCAN_LANES) void delta_scan_kernel(
     const float* __restrict__ coef, const float* __restrict__ v, float* __restrict__ state, float* __restrict__ out,
     const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, int T, int heads, int dk, int dv) {
     constexpr int SCAN_COLUMNS = COLS, SCAN_THREADS = COLS * SCAN_LANES;
     constexpr int DKP = ROWS * SCAN_LANES;                 // key rows with padding
-    constexpr int VEC = 5 * CHUNK * DKP;                   // floats of a stage's vectors
+    constexpr int NP = REMOVE ? 5 : 3;                     // vectors a token
+    constexpr int VEC = NP * CHUNK * DKP;                  // floats of a stage's vectors
     constexpr int PER_THREAD = VEC / SCAN_THREADS;
     static_assert(VEC % SCAN_THREADS == 0 && CHUNK * SCAN_COLUMNS <= SCAN_THREADS, "stage does not fit the threads");
     // stages in LDS: a ring of three for long portions, two for steps of lone tokens (less LDS, more
     // workgroups a CU); the loads that go through registers use two of them
     constexpr int NS = DEEP ? 3 : 2, AHEAD = NS - 1;
-    __shared__ __attribute__((aligned(16))) float vec[NS][5][CHUNK][DKP];
+    __shared__ __attribute__((aligned(16))) float vec[NS][NP][CHUNK][DKP];
     // a stage's values [CHUNK][COLS], in a slot of whole 64-lane loads
     constexpr int VAL_SLOT = ((CHUNK * COLS + kWave - 1) / kWave) * kWave;
     __shared__ __attribute__((aligned(16))) float val[NS][VAL_SLOT];
@@ -333,21 +345,23 @@ __global__ __launch_bounds__(COLS * SCAN_LANES) void delta_scan_kernel(
     auto work = [&](int buffer, int t0, int count) {
         // a token's vectors are read from LDS while the token before it is worked through: only the
         // state itself ties one token to the next
-        TokenRows<ROWS> rows[DEEP ? 2 : 1];
+        TokenRows<ROWS, REMOVE> rows[DEEP ? 2 : 1];
         if (DEEP) rows[0].load(&vec[buffer][0][0][0], &val[buffer][0], 0, lane, col, CHUNK * DKP, DKP, COLS);
-        auto one = [&](int tt, const TokenRows<ROWS>& now) {
+        auto one = [&](int tt, const TokenRows<ROWS, REMOVE>& now) {
             float taken = 0.f, taken2 = 0.f;
+            if constexpr (REMOVE) {
 #pragma unroll
-            for (int r = 0; r < ROWS; r += 2) {
-                taken = fmaf(now.probe[r], S[r], taken);
-                if (r + 1 < ROWS) taken2 = fmaf(now.probe[r + 1], S[r + 1], taken2);
+                for (int r = 0; r < ROWS; r += 2) {
+                    taken = fmaf(now.probe[r], S[r], taken);
+                    if (r + 1 < ROWS) taken2 = fmaf(now.probe[r + 1], S[r + 1], taken2);
+                }
+                taken = lanes16_total(taken + taken2);
             }
-            taken = lanes16_total(taken + taken2);
             float read = 0.f, read2 = 0.f;
 #pragma unroll
             for (int r = 0; r < ROWS; ++r) {
                 float s = fmaf(now.write[r], now.value, now.decay[r] * S[r]);
-                s = fmaf(-now.removal[r], taken, s);
+                if constexpr (REMOVE) s = fmaf(-now.removal[r], taken, s);
                 S[r] = s;
                 if (r & 1) read2 = fmaf(s, now.read_by[r], read2);
                 else read = fmaf(s, now.read_by[r], read);
@@ -479,21 +493,32 @@ LC_API int lc_conv_tail_update(const float* proj, int cols, int T, float* tails,
     return 0;
 }
 
-LC_API int lc_delta_scan(const float* coef, const float* v, float* state, int slots, float* out, const int* q_offsets,
-                         const int* slot_ids, int R, int T, int heads, int dk, int dv, hipStream_t stream) {
+// coef [planes, T, heads dk]: five planes (decay, probe, removal, write, read) or three (decay, write,
+// read: no removal term)
+LC_API int lc_delta_scan(const float* coef, int planes, const float* v, float* state, int slots, float* out,
+                         const int* q_offsets, const int* slot_ids, int R, int T, int heads, int dk, int dv,
+                         hipStream_t stream) {
     LC_CHECK(R >= 0 && T >= 0 && heads > 0 && dk > 0 && dv > 0 && slots >= 0, "delta_scan: bad sizes");
+    LC_CHECK(planes == 5 || planes == 3, "delta_scan: %d vectors a token are neither 5 nor 3", planes);
     LC_CHECK(dk <= DELTA_MAX_KEY, "delta_scan: heads of %d key channels are above %d", dk, DELTA_MAX_KEY);
     if (R == 0 || T == 0) return 0;
     LC_CHECK(coef && v && state && out && q_offsets && slot_ids, "delta_scan: null pointer");
     LC_CHECK(R <= 65535 && heads <= 65535, "delta_scan: too many requests or heads for the grid");
     const bool deep = T >= 16 * R;       // portions of prompts, mostly
     const dim3 grid((dv + 15) / 16, heads, R);
-#define LC_SCAN_AS(ROWS, CHUNK, DEEP, COLS)                                                                          \
-    delta_scan_kernel<ROWS, CHUNK, DEEP, COLS><<<grid, COLS * SCAN_LANES, 0, stream>>>(coef, v, state, out, q_offsets, \
-                                                                                       slot_ids, T, heads, dk, dv)
-#define LC_SCAN(ROWS, CHUNK)                          \
-    if (deep) LC_SCAN_AS(ROWS, CHUNK, true, 16);      \
-    else LC_SCAN_AS(ROWS, CHUNK, false, 16)
+#define LC_SCAN_AS(ROWS, CHUNK, DEEP, COLS, REMOVE)                                                        \
+    delta_scan_kernel<ROWS, CHUNK, DEEP, COLS, REMOVE><<<grid, COLS * SCAN_LANES, 0, stream>>>(              \
+        coef, v, state, out, q_offsets, slot_ids, T, heads, dk, dv)
+#define LC_SCAN(ROWS, CHUNK)                                            \
+    do {                                                                \
+        if (planes == 5) {                                              \
+            if (deep) LC_SCAN_AS(ROWS, CHUNK, true, 16, true);          \
+            else LC_SCAN_AS(ROWS, CHUNK, false, 16, true);              \
+        } else {                                                        \
+            if (deep) LC_SCAN_AS(ROWS, CHUNK, true, 16, false);         \
+            else LC_SCAN_AS(ROWS, CHUNK, false, 16, false);             \
+        }                                                               \
+    } while (0)
     if (dk <= 16) LC_SCAN(1, 16);
     else if (dk <= 32) LC_SCAN(2, 16);
     else if (dk <= 64) LC_SCAN(4, 16);

@@ -2,15 +2,15 @@
 // S [key, value] (float32, zeros at a sequence's start):
 //   q = silu(W_q h), k = silu(W_k h), v = silu(W_v h);   S <- decay S + k v^T;   o = S^T q
 // This file turns a step's float32 projections into the inputs of the framework's recurrence kernel
-// (S <- diag(decay) S - removal (probe^T S) + write v^T, o = S^T read), of which lightning attention is
-// the case decay = one number per head, probe = removal = 0, write = k, read = q.
+// without its removal term (S <- diag(decay) S + write v^T, o = S^T read: three vectors a token), of
+// which lightning attention is the case decay = one number per head, write = k, read = q.
 #include "common.h"
 
 namespace lc {
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
 
-// proj [T, cols]: q | k (heads x dk each) | v (heads x dv) | ...; coef [5, T, heads dk]; v_out [T, heads dv]
+// proj [T, cols]: q | k (heads x dk each) | v (heads x dv) | ...; coef [3, T, heads dk]; v_out [T, heads dv]
 __global__ void lightning_prepare_kernel(const float* __restrict__ proj, int cols, int T, int heads, int dk, int dv,
                                          const float* __restrict__ decay, float* __restrict__ coef,
                                          float* __restrict__ v_out) {
@@ -24,10 +24,8 @@ __global__ void lightning_prepare_kernel(const float* __restrict__ proj, int col
         if (c < nk) {
             const size_t at = (size_t)t * nk + c;
             coef[at] = decay[c / dk];
-            coef[plane + at] = 0.f;
-            coef[2 * plane + at] = 0.f;
-            coef[3 * plane + at] = silu_f(row[nk + c]);
-            coef[4 * plane + at] = silu_f(row[c]);
+            coef[plane + at] = silu_f(row[nk + c]);
+            coef[2 * plane + at] = silu_f(row[c]);
         } else {
             v_out[(size_t)t * nv + (c - nk)] = silu_f(row[2 * nk + (c - nk)]);
         }

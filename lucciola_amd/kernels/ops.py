@@ -98,7 +98,7 @@ _SIGNATURES = {
     "lc_general_delta_prepare": "piiiipppffppp",
     "lc_gated_delta_prepare": "piiiiiippippfpppppp",
     "lc_conv_tail_update": "piipiiippip",
-    "lc_delta_scan": "pppipppiiiiip",
+    "lc_delta_scan": "pippipppiiiiip",
     "lc_head_gate_norm": "ppiipifiiiipip",
     "lc_moe_route_logits": "pipiiippp",
     "lc_moe_combine_shared": "pppiiipipiipip",
@@ -1625,7 +1625,8 @@ def delta_scan(coef: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_offse
                slot_ids: torch.Tensor, num_requests: int, heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
     """The delta-rule recurrence over every request's tokens in order, per head:
     ``S <- diag(decay) S - removal (probe^T S) + write v^T`` (the probe meets S as the last token left it, before the decay), ``o = S^T read``.
-    ``coef`` float32 [5, T, heads key_dim] holds decay, probe, removal, write, read; ``v`` float32
+    ``coef`` float32 [5, T, heads key_dim] holds decay, probe, removal, write, read, or, for the recurrence
+    without a removal term, [3, T, heads key_dim]: decay, write, read; ``v`` float32
     [T, heads value_dim]; ``state`` float32 [slots, heads, value_dim, key_dim] (S transposed: a value
     channel's key rows lie in a row) is read at the request's slot before its first token of the step
     and written after its last.  -> float32 [T, heads value_dim]."""
@@ -1633,7 +1634,7 @@ def delta_scan(coef: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_offse
     _need(v, "delta_scan v", torch.float32, 2)
     _need(state, "delta_scan state", torch.float32, 4)
     T = v.shape[0]
-    if tuple(coef.shape) != (5, T, heads * key_dim) or v.shape[1] != heads * value_dim:
+    if coef.shape[0] not in (5, 3) or tuple(coef.shape[1:]) != (T, heads * key_dim) or v.shape[1] != heads * value_dim:
         raise KernelError("delta_scan: coef or v do not fit the heads")
     if tuple(state.shape[1:]) != (heads, value_dim, key_dim):
         raise KernelError(f"delta_scan: state {tuple(state.shape)} does not fit [slots, {heads}, {value_dim}, {key_dim}]")
@@ -1644,7 +1645,7 @@ def delta_scan(coef: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_offse
     check_delta_sizes("delta_scan", key_dim, value_dim)
     out = torch.empty((T, heads * value_dim), dtype=torch.float32, device=v.device)
     if T:
-        _call("lc_delta_scan", _ptr(coef), _ptr(v), _ptr(state), state.shape[0], _ptr(out), _ptr(q_offsets),
+        _call("lc_delta_scan", _ptr(coef), coef.shape[0], _ptr(v), _ptr(state), state.shape[0], _ptr(out), _ptr(q_offsets),
               _ptr(slot_ids), num_requests, T, heads, key_dim, value_dim, _stream())
     return out
 
@@ -1721,15 +1722,15 @@ def moe_combine_shared(y: torch.Tensor, routing: Routing, shared: torch.Tensor, 
 # ------------------------------------------------------------------------------ lightning attention
 def lightning_prepare(proj: torch.Tensor, heads: int, key_dim: int, value_dim: int, decay: torch.Tensor):
     """The scan's inputs of lightning attention from the float32 projections ``proj`` [T, >= heads (2 key_dim
-    + value_dim)]: columns q | k | v.  Returns ``coef`` float32 [5, T, heads key_dim] (decay = ``decay``[head]
-    in every channel, probe = removal = 0, write = silu(k), read = silu(q)) and ``v`` = silu(v) float32
+    + value_dim)]: columns q | k | v.  Returns ``coef`` float32 [3, T, heads key_dim] (decay = ``decay``[head]
+    in every channel, write = silu(k), read = silu(q): no removal term) and ``v`` = silu(v) float32
     [T, heads value_dim]."""
     _need(proj, "lightning proj", torch.float32, 2)
     _need(decay, "lightning decay", torch.float32, 1)
     T = proj.shape[0]
     if proj.shape[1] < heads * (2 * key_dim + value_dim) or decay.shape[0] != heads:
         raise KernelError(f"lightning_prepare: proj {tuple(proj.shape)} or decay do not fit {heads} heads")
-    coef = torch.empty((5, T, heads * key_dim), dtype=torch.float32, device=proj.device)
+    coef = torch.empty((3, T, heads * key_dim), dtype=torch.float32, device=proj.device)
     v = torch.empty((T, heads * value_dim), dtype=torch.float32, device=proj.device)
     if T:
         _call("lc_lightning_prepare", _ptr(proj), proj.shape[1], T, heads, key_dim, value_dim, _ptr(decay), _ptr(coef),

@@ -310,10 +310,10 @@ def lightning_prepare(proj, heads, key_dim, value_dim, decay):
     def silu(z):
         return z * torch.sigmoid(z)
     p = proj.to(F64)
-    coef = torch.zeros(5, T, nk, dtype=F64)
+    coef = torch.zeros(3, T, nk, dtype=F64)       # decay, write, read: the recurrence without removal
     coef[0] = decay.to(F64).repeat_interleave(key_dim)[None, :]
-    coef[3] = silu(p[:, nk:2 * nk])
-    coef[4] = silu(p[:, :nk])
+    coef[1] = silu(p[:, nk:2 * nk])
+    coef[2] = silu(p[:, :nk])
     return coef.to(torch.float32), silu(p[:, 2 * nk:2 * nk + nv]).to(torch.float32)
 
 
@@ -495,6 +495,9 @@ def conv_tail_update(proj, tail, channels, num_taps, q_offsets, slot_ids, num_re
 
 def delta_scan(coef, v, state, q_offsets, slot_ids, num_requests, heads, key_dim, value_dim):
     T = v.shape[0]
+    if coef.shape[0] == 3:      # decay, write, read: no removal term
+        zero = torch.zeros_like(coef[0])
+        coef = torch.stack([coef[0], zero, zero, coef[1], coef[2]])
     c = coef.to(F64).view(5, T, heads, key_dim)
     vv = v.to(F64).view(T, heads, value_dim)
     out = torch.zeros(T, heads, value_dim, dtype=F64)
