@@ -207,10 +207,16 @@ def test_a_negative_choice_score_inside_a_kept_group_wins():
 
 
 @pytest.mark.parametrize("heads,dk,dv,lengths", [(2, 16, 16, [5, 1, 40]), (3, 7, 9, [1, 1, 1, 1]), (2, 32, 64, [70]),
-                                                 (1, 128, 128, [33, 2]), (4, 48, 40, [9])])
+                                                 (1, 128, 128, [33, 2]), (4, 48, 40, [9]),
+                                                 # every key size whose stages load straight into LDS, in long
+                                                 # portions (several stages, a last one that is not full) and in
+                                                 # steps of lone tokens
+                                                 (3, 16, 24, [90, 2]), (2, 32, 8, [150]), (2, 64, 48, [100, 1, 1]),
+                                                 (1, 256, 32, [37]), (2, 256, 20, [1, 1, 1]), (2, 128, 16, [1, 1, 1, 1]),
+                                                 (2, 64, 16, [1, 1])])
 def test_lightning_kernels_against_the_recurrence(heads, dk, dv, lengths):
-    """Projections -> scan inputs -> scan -> gated read-out over two steps, against the token-by-token
-    recurrence written out."""
+    """Projections -> scan inputs -> scan (its form without a removal term) -> gated read-out over two
+    steps, against the token-by-token recurrence written out."""
     g = torch.Generator().manual_seed(heads * dk)
     decay = torch.tensor([0.5, 0.9, 0.99, 1.0][:heads])
     slots = [2, 0, 3, 1][:len(lengths)]
