@@ -121,6 +121,30 @@ class PagedLatent(CacheNeed):
 
 
 @dataclass(frozen=True)
+class PagedRows(CacheNeed):
+    """A row of keys and a row of values per token, in pages, the two of widths of their own (key heads and
+    value heads of different numbers or sizes, several key maps that share a value).  ``window`` as for
+    :class:`PagedKV`.
+
+    Memory per site, token-major: keys ``[pages, page, key_width]``, values ``[pages, page, value_width]``; any
+    page size."""
+
+    key_width: int
+    value_width: int
+    window: Optional[int] = None
+
+    paged = True
+
+    def bytes_per_page(self, page_size: int, dtype: torch.dtype) -> int:
+        return page_size * (self.key_width + self.value_width) * _element_size(dtype)
+
+    def allocate(self, layout: CacheLayout, dtype: torch.dtype, device):
+        pages, page = layout.kernel_pages, layout.kernel_page
+        return (torch.zeros((pages, page, self.key_width), dtype=dtype, device=device),
+                torch.zeros((pages, page, self.value_width), dtype=dtype, device=device))
+
+
+@dataclass(frozen=True)
 class FixedState(CacheNeed):
     """A tensor of fixed shape per live request: ``[max_seqs, *shape]``, indexed by the
     request's slot and zeroed when a request starts."""

@@ -34,10 +34,11 @@ __device__ __forceinline__ void row_moments(const float* row, int n, float eps, 
 }
 
 // One workgroup per output row r; src row = rows ? rows[r] : r.
-//   d = delta[src], layer-normed with (pw, pb, peps) if pw;  v = h ? h[src] + d : d
+//   d = delta[src], layer-normed with (pw, pb, peps) if pw;  v = h ? h[src] + dscale d : d
 //   if (write_h) h[src] = v;  out[r] = w ? layer norm of v with (w, b, eps) : v
 template <typename TD, typename TO>
-__global__ void layer_norm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ pw,
+__global__ void layer_norm_kernel(float* __restrict__ h, const TD* __restrict__ delta, float dscale,
+                                  const float* __restrict__ pw,
                                   const float* __restrict__ pb, float peps, const int* __restrict__ rows,
                                   const float* __restrict__ w, const float* __restrict__ b, float eps,
                                   TO* __restrict__ out, int n, int write_h) {
@@ -58,7 +59,7 @@ __global__ void layer_norm_kernel(float* __restrict__ h, const TD* __restrict__ 
     if (h) {
         float* hr = h + src * n;
         for (int i = threadIdx.x; i < n; i += blockDim.x) {     // a thread meets its own entries only
-            const float v = delta ? hr[i] + row[i] : hr[i];
+            const float v = delta ? fmaf(dscale, row[i], hr[i]) : hr[i];
             row[i] = v;
             if (write_h) hr[i] = v;
         }
@@ -76,7 +77,7 @@ __global__ void layer_norm_kernel(float* __restrict__ h, const TD* __restrict__ 
 // The same for rows of up to ITEMS entries a thread: every operand is asked for before the first
 // sum, so a row costs one trip to memory and not one per stage.
 template <typename TD, typename TO, int ITEMS>
-__global__ void layer_norm_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+__global__ void layer_norm_rows_kernel(float* __restrict__ h, const TD* __restrict__ delta, float dscale,
                                        const float* __restrict__ pw, const float* __restrict__ pb, float peps,
                                        const int* __restrict__ rows, const float* __restrict__ w,
                                        const float* __restrict__ b, float eps, TO* __restrict__ out, int n,
@@ -116,7 +117,7 @@ __global__ void layer_norm_rows_kernel(float* __restrict__ h, const TD* __restri
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
         const int i = tid + k * step;
-        const float v = h ? (delta ? hv[k] + d[k] : hv[k]) : d[k];
+        const float v = h ? (delta ? fmaf(dscale, d[k], hv[k]) : hv[k]) : d[k];
         d[k] = i < n ? v : 0.f;
         if (h && delta && write_h && i < n) h[src * n + i] = v;
         s += d[k];
@@ -250,7 +251,7 @@ using namespace lc;
 
 // h float32 [T, n] or null; delta [T, n] of dtype dt_delta or null; (pw, pb, peps): the branch's own
 // norm or null; rows int32 [R] or null; (w, b, eps): the norm of the sum, or null to leave it as it is
-LC_API int lc_layer_norm(float* h, const void* delta, int dt_delta, const float* pw, const float* pb, float peps,
+LC_API int lc_layer_norm(float* h, const void* delta, int dt_delta, float dscale, const float* pw, const float* pb, float peps,
                          const int* rows, const float* w, const float* b, float eps, void* out, int dt_out, int R,
                          int n, int write_h, int T, hipStream_t stream) {
     LC_CHECK(R >= 0 && n > 0 && T >= 0, "layer_norm: bad sizes R=%d n=%d", R, n);
@@ -267,10 +268,10 @@ LC_API int lc_layer_norm(float* h, const void* delta, int dt_delta, const float*
     const size_t lds = (size_t)n * sizeof(float);
 #define LC_LN(TD, TO)                                                                                           \
     if (in_registers)                                                                                           \
-        layer_norm_rows_kernel<TD, TO, ITEMS><<<R, threads, 0, stream>>>(h, (const TD*)delta, pw, pb, peps, rows, w, \
+        layer_norm_rows_kernel<TD, TO, ITEMS><<<R, threads, 0, stream>>>(h, (const TD*)delta, dscale, pw, pb, peps, rows, w, \
                                                                          b, eps, (TO*)out, n, write_h);         \
     else                                                                                                        \
-        layer_norm_kernel<TD, TO><<<R, threads, lds, stream>>>(h, (const TD*)delta, pw, pb, peps, rows, w, b, eps, \
+        layer_norm_kernel<TD, TO><<<R, threads, lds, stream>>>(h, (const TD*)delta, dscale, pw, pb, peps, rows, w, b, eps, \
                                                                (TO*)out, n, write_h)
     const int dd = delta ? dt_delta : DT_F32;
     if (dd == DT_F32 && dt_out == DT_F32) LC_LN(float, float);

@@ -11,6 +11,7 @@
 // A sorted row's value does not depend on where in its expert's stretch it lies, so the order in
 // which the pairs of one expert arrive (atomic counters) changes no result.
 #include "common.h"
+#include "activations.h"
 
 namespace lc {
 
@@ -237,25 +238,63 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, const float* __r
     }
 }
 
-// the same plus sigmoid(gates[t, gate_column]) * shared[t]
+// the same plus sigmoid(gates[t, gate_column]) * shared[t]; weights null: every choice counts 1; gates null: the
+// shared rows count 1
 template <typename T, typename TS>
 __global__ void moe_combine_shared_kernel(const float* __restrict__ y, const float* __restrict__ weights,
                                           const int* __restrict__ entry_row, int top, int n,
                                           const TS* __restrict__ shared, const float* __restrict__ gates, int gate_cols,
                                           int gate_column, T* __restrict__ out) {
     const int t = blockIdx.x;
-    const float g = 1.f / (1.f + expf(-gates[(size_t)t * gate_cols + gate_column]));
+    const float g = gates ? 1.f / (1.f + expf(-gates[(size_t)t * gate_cols + gate_column])) : 1.f;
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         float total = 0.f;
         for (int k = 0; k < top; ++k)
-            total = fmaf(weights[(size_t)t * top + k], y[(size_t)entry_row[(size_t)t * top + k] * n + i], total);
-        out[(size_t)t * n + i] = from_f32<T>(fmaf(g, to_f32(shared[(size_t)t * n + i]), total));
+            total = fmaf(weights ? weights[(size_t)t * top + k] : 1.f, y[(size_t)entry_row[(size_t)t * top + k] * n + i], total);
+        out[(size_t)t * n + i] = from_f32<T>(shared ? fmaf(g, to_f32(shared[(size_t)t * n + i]), total) : total);
+    }
+}
+
+// Sorted row entry_row[e] of entry e (a token's choice): act(w gate) * (w up) with w = weights[e], which is what
+// the gated expert makes of w times its input (both products are linear).  gu [rows, 2 I] -> out [rows, I]
+template <typename T>
+__global__ void gated_activation_weighted_kernel(const T* __restrict__ gu, T* __restrict__ out,
+                                                 const float* __restrict__ weights, const int* __restrict__ entry_row,
+                                                 int I, int kind, size_t total) {
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t e = idx / I, i = idx % I;
+        const size_t row = (size_t)entry_row[e];
+        const float w = weights[e];
+        const float g = w * to_f32(gu[row * 2 * I + i]), u = w * to_f32(gu[row * 2 * I + I + i]);
+        out[row * I + i] = from_f32<T>((kind == 0 ? g * sigmoid(g) : activate(g, ACT_GELU_TANH)) * u);
     }
 }
 
 }  // namespace lc
 
 using namespace lc;
+
+// gu [entries, 2 I] (sorted rows) -> out [entries, I]; weights float32 [entries], entry_row int32 [entries];
+// kind 0: silu, 1: gelu (tanh form)
+LC_API int lc_gated_activation_weighted(const void* gu, void* out, int dt, const float* weights, const int* entry_row,
+                                        int entries, int I, int kind, hipStream_t stream) {
+    LC_CHECK(entries >= 0 && I > 0 && (kind == 0 || kind == 1), "gated_activation_weighted: bad arguments");
+    if (entries == 0) return 0;
+    LC_CHECK(gu && out && weights && entry_row, "gated_activation_weighted: null pointer");
+    const size_t total = (size_t)entries * I;
+    const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    if (dt == DT_F32)
+        gated_activation_weighted_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, weights,
+                                                                            entry_row, I, kind, total);
+    else if (dt == DT_BF16)
+        gated_activation_weighted_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, weights, entry_row,
+                                                                           I, kind, total);
+    else
+        LC_CHECK(false, "gated_activation_weighted: unknown dtype %d", dt);
+    LC_LAUNCH_CHECK("gated_activation_weighted");
+    return 0;
+}
 
 LC_API int lc_moe_max_experts(void) { return MOE_MAX_EXPERTS; }
 
@@ -318,10 +357,10 @@ LC_API int lc_moe_route_logits(const float* logits, int cols, const float* bias,
 LC_API int lc_moe_combine_shared(const float* y, const float* weights, const int* entry_row, int T, int top, int n,
                                  const void* shared, int dt_shared, const float* gates, int gate_cols, int gate_column,
                                  void* out, int dt, hipStream_t stream) {
-    LC_CHECK(T >= 0 && top > 0 && n > 0 && gate_cols > 0 && gate_column >= 0 && gate_column < gate_cols,
+    LC_CHECK(T >= 0 && top > 0 && n > 0 && (!gates || (gate_cols > 0 && gate_column >= 0 && gate_column < gate_cols)),
              "moe combine: bad sizes");
     if (T == 0) return 0;
-    LC_CHECK(y && weights && entry_row && shared && gates && out, "moe combine: null pointer");
+    LC_CHECK(y && entry_row && out && (shared || !gates), "moe combine: null pointer");
     const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
 #define LC_COMBINE(TO, TS)                                                                                       \
     moe_combine_shared_kernel<TO, TS><<<T, threads, 0, stream>>>(y, weights, entry_row, top, n, (const TS*)shared, \

@@ -100,6 +100,12 @@ class SiteView:
         return SiteView(self.batch, self.index, self.writes_cache, self.caches[k:k + 1],
                         self.page_views[k:k + 1])
 
+    def span(self, first: int, count: int) -> "SiteView":
+        """The view of ``count`` needs from the ``first`` on: what a part that is made of parts hands to the one
+        of them whose needs these are."""
+        return SiteView(self.batch, self.index, self.writes_cache, self.caches[first:first + count],
+                        self.page_views[first:first + count])
+
 
 @dataclass
 class StepBatch:

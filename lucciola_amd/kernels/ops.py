@@ -91,7 +91,7 @@ _SIGNATURES = {
     "lc_lightning_readout": "ppiipfiipip",
     "lc_moe_lists": "piiiippppp",
     "lc_moe_combine": "pppiiipip",
-    "lc_layer_norm": "ppippfpppfpiiiiip",
+    "lc_layer_norm": "ppifppfpppfpiiiiip",
     "lc_embedding_sinusoid": "pppippiiifp",
     "lc_gated_activation": "ppiiiip",
     "lc_head_norm_write": "piiiiiiippfpppppiip",
@@ -102,6 +102,12 @@ _SIGNATURES = {
     "lc_head_gate_norm": "ppiipifiiiipip",
     "lc_moe_route_logits": "pipiiippp",
     "lc_moe_combine_shared": "pppiiipipiipip",
+    "lc_gated_activation_weighted": "ppippiiip",
+    "lc_masked_attention": "pppi" + "ppp" + "ii" + "i" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
+    "lc_attention_prepare": "p" + "iiiiiii" + "pip" + "ppp" + "pip" + "if" + "ppp" + "i" + "pp",
+    "lc_state_space_prepare": "piiiiii" + "ppi" + "ppp" + "ppp" + "pp" + "p",
+    "lc_state_space_readout": "pppiipiipifipip",
+    "lc_scaled_sum": "pifpifpqp",
 }
 
 
@@ -1386,9 +1392,9 @@ class NormedBranch:
 
 
 def layer_norm(h: torch.Tensor, delta, weight: torch.Tensor, bias: torch.Tensor, eps: float,
-               out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+               out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, branch_scale: float = 1.0) -> torch.Tensor:
     """Layer norm ``(v - mean) / sqrt(var + eps) * weight + bias`` of the float32 residual stream ``h``
-    [T, n] with the pending addition ``delta`` taken in first (v = h + delta); ``delta`` may be a
+    [T, n] with the pending addition ``delta`` taken in first (v = h + branch_scale delta); ``delta`` may be a
     :class:`NormedBranch`, which is normed with its own weights before it is added.  Without ``rows``:
     ``h`` becomes v in place and every row is normed; with ``rows`` (int32 [R]): only those rows, ``h``
     stays as it is."""
@@ -1417,7 +1423,8 @@ def layer_norm(h: torch.Tensor, delta, weight: torch.Tensor, bias: torch.Tensor,
     R = T if rows is None else rows.shape[0]
     out = torch.empty((R, n), dtype=out_dtype, device=h.device)
     if R:
-        _call("lc_layer_norm", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, _ptr(post_w),
+        _call("lc_layer_norm", _ptr(h), _ptr(delta), _dt(delta) if delta is not None else DT_F32, float(branch_scale),
+              _ptr(post_w),
               _ptr(post_b), float(post_eps), _ptr(rows), _ptr(weight), _ptr(bias), float(eps), _ptr(out), _dt(out),
               R, n, 1 if (rows is None and delta is not None) else 0, T, _stream())
     return out
@@ -1434,7 +1441,7 @@ def layer_norm_act(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, ep
     out = torch.empty_like(x)
     rows = x.numel() // n
     if rows:
-        _call("lc_layer_norm", None, _ptr(x), _dt(x), _ptr(weight), _ptr(bias), float(eps), None, None, None,
+        _call("lc_layer_norm", None, _ptr(x), _dt(x), 1.0, _ptr(weight), _ptr(bias), float(eps), None, None, None,
               0.0, _ptr(out), _dt(out), rows, n, 0, rows, _stream())
     return out
 
@@ -1470,6 +1477,21 @@ def gated_activation(gu: torch.Tensor, kind: str) -> torch.Tensor:
     out = torch.empty((T, two_i // 2), dtype=gu.dtype, device=gu.device)
     if T:
         _call("lc_gated_activation", _ptr(gu), _ptr(out), _dt(gu), T, two_i // 2, GATE_ACTIVATIONS[kind], _stream())
+    return out
+
+
+def gated_activation_weighted(gu: torch.Tensor, kind: str, routing: "Routing") -> torch.Tensor:
+    """As :func:`gated_activation` over the experts' sorted rows, each row's gate and up entries first times
+    the weight of its (token, choice) pair: ``act(w gate) * (w up)``, which is what a gated expert makes of
+    w times its input."""
+    _need(gu, "gated_activation_weighted input", None, 2)
+    rows, two_i = gu.shape
+    if two_i % 2 or rows != routing.entry_row.shape[0]:
+        raise KernelError("gated_activation_weighted: the rows do not fit the routing")
+    out = torch.empty((rows, two_i // 2), dtype=gu.dtype, device=gu.device)
+    if rows:
+        _call("lc_gated_activation_weighted", _ptr(gu), _ptr(out), _dt(gu), _ptr(routing.weights),
+              _ptr(routing.entry_row), rows, two_i // 2, GATE_ACTIVATIONS[kind], _stream())
     return out
 
 
@@ -1702,20 +1724,28 @@ def moe_route_logits(logits: torch.Tensor, experts: int, top: int, bias: Optiona
     return Routing(ids, weights, row_start, tile_start, sorted_token, entry_row, E, tile, (T * top) // tile + E)
 
 
-def moe_combine_shared(y: torch.Tensor, routing: Routing, shared: torch.Tensor, gates: torch.Tensor,
-                       gate_column: int, out_dtype: torch.dtype) -> torch.Tensor:
-    """:func:`moe_combine` plus ``sigmoid(gates[t, gate_column]) * shared[t]`` (``gates`` float32)."""
+def moe_combine_shared(y: torch.Tensor, routing: Routing, shared: Optional[torch.Tensor],
+                       gates: Optional[torch.Tensor], gate_column: int, out_dtype: torch.dtype,
+                       weighted: bool = True) -> torch.Tensor:
+    """:func:`moe_combine` plus ``sigmoid(gates[t, gate_column]) * shared[t]`` (``gates`` float32; without
+    ``gates`` the shared rows count as they are, without ``shared`` there are none).  Not ``weighted``: every
+    choice counts 1 (the weights have been applied on the experts' way in)."""
     _need(y, "moe_combine_shared y", torch.float32, 2)
-    _need(shared, "moe_combine_shared shared", None, 2)
-    _need(gates, "moe_combine_shared gates", torch.float32, 2)
     T, top = routing.ids.shape
     n = y.shape[1]
-    if y.shape[0] != T * top or tuple(shared.shape) != (T, n) or gates.shape[0] != T or not 0 <= gate_column < gates.shape[1]:
+    if shared is not None:
+        _need(shared, "moe_combine_shared shared", None, 2)
+    if gates is not None:
+        _need(gates, "moe_combine_shared gates", torch.float32, 2)
+        if shared is None or gates.shape[0] != T or not 0 <= gate_column < gates.shape[1]:
+            raise KernelError("moe_combine_shared: the gates do not fit the rows")
+    if y.shape[0] != T * top or (shared is not None and tuple(shared.shape) != (T, n)):
         raise KernelError("moe_combine_shared: the operands do not fit the routing")
     out = torch.empty((T, n), dtype=out_dtype, device=y.device)
     if T:
-        _call("lc_moe_combine_shared", _ptr(y), _ptr(routing.weights), _ptr(routing.entry_row), T, top, n,
-              _ptr(shared), _dt(shared), _ptr(gates), gates.shape[1], gate_column, _ptr(out), _dt(out), _stream())
+        _call("lc_moe_combine_shared", _ptr(y), _ptr(routing.weights if weighted else None), _ptr(routing.entry_row),
+              T, top, n, _ptr(shared), _dt(shared) if shared is not None else DT_F32, _ptr(gates),
+              gates.shape[1] if gates is not None else 0, gate_column, _ptr(out), _dt(out), _stream())
     return out
 
 
@@ -1753,4 +1783,183 @@ def lightning_readout(o: torch.Tensor, gates: torch.Tensor, gate_column: int, we
     if T:
         _call("lc_lightning_readout", _ptr(o), _ptr(gates), gates.shape[1], gate_column, _ptr(weight), float(eps), T, n,
               _ptr(out), _dt(out), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ masked attention
+MASKED_ATTENTION_MAX = 256      # entries of a key head and of a value head at most
+SHORT_CONV_MAX_TAPS = 8
+
+
+def attention_prepare(proj: torch.Tensor, nq: int, nk: int, nv: int, d: int, dv: int, out_dtype: torch.dtype,
+                      k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                      rows: Optional[torch.Tensor], taps: Optional[torch.Tensor] = None,
+                      tail: Optional[torch.Tensor] = None, tok_req: Optional[torch.Tensor] = None,
+                      q_offsets: Optional[torch.Tensor] = None, slot_ids: Optional[torch.Tensor] = None,
+                      table: Optional[torch.Tensor] = None, rot: int = 0,
+                      positions: Optional[torch.Tensor] = None, unit_eps: Optional[float] = None) -> torch.Tensor:
+    """q, k and v of a step from the first (nq + nk) d + nv dv columns of the float32 projections ``proj`` (q heads
+    | k heads | v heads).  ``taps`` float32 [columns, K]: every column first passes a causal convolution over time whose
+    inputs from before the step come from ``tail`` float32 [slots, K - 1, columns] (the request's last K - 1
+    inputs, oldest first).  ``table`` float32 [positions, rot] (cosines | sines): entries 2i, 2i + 1 of the first
+    ``rot`` of every q and k head are rotated by angle i of the token's position.  ``unit_eps``: every q and k
+    head is divided by its root mean square.  Returns q [T, nq d] of ``out_dtype``; k and v go to row ``rows[t]``
+    of ``k_cache`` [rows, nk d] and ``v_cache`` [rows, nv dv] (where ``rows`` is given and not negative)."""
+    _need(proj, "attention_prepare proj", torch.float32, 2)
+    T, cols = proj.shape
+    C = (nq + nk) * d + nv * dv
+    if cols < C:
+        raise KernelError(f"attention_prepare: proj has {cols} columns, fewer than the heads' {C}")
+    if max(d, dv) > MASKED_ATTENTION_MAX:
+        raise KernelError(f"attention_prepare: heads of {d}/{dv} entries are above {MASKED_ATTENTION_MAX}")
+    K = 0
+    if taps is not None:
+        _need(taps, "conv taps", torch.float32, 2)
+        K = taps.shape[1]
+        if taps.shape[0] != C or not 1 <= K <= SHORT_CONV_MAX_TAPS:
+            raise KernelError(f"attention_prepare: taps {tuple(taps.shape)} do not fit {C} columns")
+        for t, what in ((tok_req, "tok_req"), (q_offsets, "q_offsets"), (slot_ids, "slot_ids")):
+            _need(t, what, torch.int32, 1)
+        if K > 1:
+            _need(tail, "conv tail", torch.float32, 3)
+            if tuple(tail.shape[1:]) != (K - 1, C):
+                raise KernelError("attention_prepare: the tail does not fit the taps")
+    if table is not None:
+        _need(table, "rotary table", torch.float32, 2)
+        _need(positions, "positions", torch.int32, 1)
+        if table.shape[1] != rot or rot % 2 or rot > d:
+            raise KernelError(f"attention_prepare: a table of {table.shape[1]} columns for {rot} rotated entries of {d}")
+    if rows is not None:
+        _need(rows, "cache rows", torch.int32, 1)
+        if k_cache is None or v_cache is None or k_cache.dtype != out_dtype or v_cache.dtype != out_dtype:
+            raise KernelError("attention_prepare: the cache must have the queries' dtype")
+        if k_cache.shape[-1] != nk * d or v_cache.shape[-1] != nv * dv:
+            raise KernelError("attention_prepare: the cache rows do not fit the heads")
+    q = torch.empty((T, nq * d), dtype=out_dtype, device=proj.device)
+    if T:
+        _call("lc_attention_prepare", _ptr(proj), cols, T, nq, nk, nv, d, dv, _ptr(taps), K, _ptr(tail),
+              _ptr(tok_req), _ptr(q_offsets), _ptr(slot_ids), _ptr(table), int(rot), _ptr(positions),
+              0 if unit_eps is None else 1, float(unit_eps or 0.0), _ptr(q), _ptr(k_cache if rows is not None else None),
+              _ptr(v_cache if rows is not None else None), _dt(q), _ptr(rows), _stream())
+    return q
+
+
+def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, tok_req: torch.Tensor,
+                     positions: torch.Tensor, block_table: torch.Tensor, page_size: int, heads: int, kv_heads: int,
+                     maps: int, d: int, dv: int, scale: float, chunk: int = 0, window: int = 0,
+                     r1: Optional[torch.Tensor] = None, r2: Optional[torch.Tensor] = None,
+                     sink: Optional[torch.Tensor] = None, subtract: float = 0.0, unit_eps: Optional[float] = None,
+                     out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, gate_column: int = 0) -> torch.Tensor:
+    """Attention of every token of the batch over its request's cached keys lo .. p (p its position; lo the start
+    of its chunk of ``chunk`` positions, of its window of ``window``, or 0), float32 arithmetic.  ``q`` [T, heads
+    maps d]; ``k_cache`` [pages, page, kv_heads maps d], ``v_cache`` [pages, page, kv_heads dv].  Scores are
+    ``scale`` (q . k) minus ``r1[h] ln(1 + r2[h] (p - j))`` where the bias is given; ``sink`` float32 [heads] adds
+    exp(sink[h]) to the softmax's denominator.  ``maps`` = 2: a head's two maps over the same values are combined as
+    a_0 - ``subtract`` a_1.  ``unit_eps``: the head's output is divided by its root mean square and multiplied by
+    ``out_scale``.  ``gate`` float32 [T, >= gate_column + heads dv]: the output times sigmoid of those columns.
+    -> [T, heads dv] in q's dtype."""
+    _need(q, "masked_attention q", None, 2)
+    T = q.shape[0]
+    if q.shape[1] != heads * maps * d:
+        raise KernelError(f"masked_attention: q has {q.shape[1]} columns, expected {heads * maps * d}")
+    for cache, width, what in ((k_cache, kv_heads * maps * d, "keys"), (v_cache, kv_heads * dv, "values")):
+        _need(cache, f"masked_attention {what}", q.dtype, 3)
+        if cache.shape[1] != page_size or cache.shape[2] != width:
+            raise KernelError(f"masked_attention: the {what} {tuple(cache.shape)} do not fit pages of {page_size} "
+                              f"rows of {width}")
+    _need(tok_req, "tok_req", torch.int32, 1)
+    _need(positions, "positions", torch.int32, 1)
+    _need(block_table, "block_table", torch.int32, 2)
+    for vec, what in ((r1, "r1"), (r2, "r2"), (sink, "sink")):
+        if vec is not None:
+            _need(vec, f"masked_attention {what}", torch.float32, 1)
+            if vec.shape[0] != heads:
+                raise KernelError(f"masked_attention: {what} has {vec.shape[0]} entries for {heads} heads")
+    if gate is not None:
+        _need(gate, "masked_attention gate", torch.float32, 2)
+        if gate.shape[0] != T or gate_column < 0 or gate_column + heads * dv > gate.shape[1]:
+            raise KernelError("masked_attention: the gate does not fit the rows")
+    out = torch.empty((T, heads * dv), dtype=q.dtype, device=q.device)
+    if T:
+        _call("lc_masked_attention", _ptr(q), _ptr(k_cache), _ptr(v_cache), _dt(q), _ptr(tok_req), _ptr(positions),
+              _ptr(block_table), block_table.shape[1], int(page_size), T, heads, kv_heads, maps, d, dv, float(scale),
+              int(chunk), int(window), _ptr(r1), _ptr(r2), _ptr(sink), float(subtract), 0 if unit_eps is None else 1,
+              float(unit_eps or 0.0), float(out_scale), _ptr(gate), gate.shape[1] if gate is not None else 0,
+              int(gate_column), _ptr(out), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------ the state-space mixer
+def state_space_prepare(proj: torch.Tensor, heads: int, groups: int, state: int, value_dim: int, taps: torch.Tensor,
+                        bias: torch.Tensor, tail: Optional[torch.Tensor], dt_bias: torch.Tensor, a_log: torch.Tensor,
+                        tok_req: torch.Tensor, q_offsets: torch.Tensor, slot_ids: torch.Tensor):
+    """The scan's inputs of the state-space mixer from the float32 projections ``proj`` [T, 2 heads value_dim + 2
+    groups state + heads]: columns x | B | C | z | dt.  x, B and C pass the convolution ``taps`` [C, K] (+ ``bias``,
+    then SiLU; inputs from before the step from ``tail`` [slots, K - 1, C]).  step = softplus(dt + dt_bias).
+    Returns ``coef`` float32 [3, T, heads state] (decay = exp(-exp(a_log) step) in every channel, write = step B,
+    read = C, each head with its group's B and C) and x float32 [T, heads value_dim]."""
+    _need(proj, "state_space proj", torch.float32, 2)
+    T = proj.shape[0]
+    inner = heads * value_dim
+    C = inner + 2 * groups * state
+    if proj.shape[1] != C + inner + heads or heads % groups:
+        raise KernelError(f"state_space_prepare: proj has {proj.shape[1]} columns, expected {C + inner + heads}")
+    _need(taps, "conv taps", torch.float32, 2)
+    _need(bias, "conv bias", torch.float32, 1)
+    K = taps.shape[1]
+    if taps.shape[0] != C or bias.shape[0] != C or not 1 <= K <= SHORT_CONV_MAX_TAPS:
+        raise KernelError("state_space_prepare: taps or bias do not fit the channels")
+    if K > 1:
+        _need(tail, "conv tail", torch.float32, 3)
+        if tuple(tail.shape[1:]) != (K - 1, C):
+            raise KernelError("state_space_prepare: the tail does not fit the taps")
+    for vec, what in ((dt_bias, "dt_bias"), (a_log, "a_log")):
+        _need(vec, what, torch.float32, 1)
+        if vec.shape[0] != heads:
+            raise KernelError(f"state_space_prepare: {what} has {vec.shape[0]} entries for {heads} heads")
+    for t, what in ((tok_req, "tok_req"), (q_offsets, "q_offsets"), (slot_ids, "slot_ids")):
+        _need(t, what, torch.int32, 1)
+    if tok_req.shape[0] != T:
+        raise KernelError("state_space_prepare: the token map does not fit")
+    coef = torch.empty((3, T, heads * state), dtype=torch.float32, device=proj.device)
+    x = torch.empty((T, inner), dtype=torch.float32, device=proj.device)
+    if T:
+        _call("lc_state_space_prepare", _ptr(proj), proj.shape[1], T, heads, groups, state, value_dim, _ptr(taps),
+              _ptr(bias), K, _ptr(tail if K > 1 else None), _ptr(dt_bias), _ptr(a_log), _ptr(tok_req), _ptr(q_offsets),
+              _ptr(slot_ids), _ptr(coef), _ptr(x), _stream())
+    return coef, x
+
+
+def state_space_readout(o: torch.Tensor, x: torch.Tensor, gates: torch.Tensor, z_column: int, skip: torch.Tensor,
+                        heads: int, value_dim: int, weight: torch.Tensor, parts: int, eps: float,
+                        out_dtype: torch.dtype) -> torch.Tensor:
+    """``(o + skip[head] x) silu(z)`` with z the float32 columns ``z_column`` .. + n of ``gates``, the row divided by
+    its root mean square in ``parts`` equal parts (eps inside the root), times ``weight`` [n].  -> [T, n]."""
+    _need(o, "state_space_readout o", torch.float32, 2)
+    _need(x, "state_space_readout x", torch.float32, 2)
+    _need(gates, "state_space_readout gates", torch.float32, 2)
+    _need(skip, "state_space_readout skip", torch.float32, 1)
+    _need(weight, "state_space_readout weight", torch.float32, 1)
+    T, n = o.shape
+    if n != heads * value_dim or tuple(x.shape) != (T, n) or gates.shape[0] != T or z_column < 0 \
+            or z_column + n > gates.shape[1] or skip.shape[0] != heads or weight.shape[0] != n or parts < 1 or n % parts:
+        raise KernelError("state_space_readout: the operands do not fit the heads")
+    out = torch.empty((T, n), dtype=out_dtype, device=o.device)
+    if T:
+        _call("lc_state_space_readout", _ptr(o), _ptr(x), _ptr(gates), gates.shape[1], int(z_column), _ptr(skip), heads,
+              value_dim, _ptr(weight), int(parts), float(eps), T, _ptr(out), _dt(out), _stream())
+    return out
+
+
+def scaled_sum(a, a_scale: float, b, b_scale: float) -> torch.Tensor:
+    """``a_scale a + b_scale b`` as float32 (two branches that a layer adds to its stream as one)."""
+    a, b = value(a), value(b)
+    _need(a, "scaled_sum a", None, 2)
+    _need(b, "scaled_sum b", None, 2)
+    if a.shape != b.shape:
+        raise KernelError(f"scaled_sum: {tuple(a.shape)} and {tuple(b.shape)} differ")
+    out = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    if out.numel():
+        _call("lc_scaled_sum", _ptr(a), _dt(a), float(a_scale), _ptr(b), _dt(b), float(b_scale), _ptr(out),
+              out.numel(), _stream())
     return out

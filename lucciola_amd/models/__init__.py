@@ -1,2 +1,2 @@
 """Architectures: importing this package registers them."""
-from . import kikunex, larupel, pubodra, qwen3  # noqa: F401
+from . import kikunex, larupel, pubodra, qwen3, rununex  # noqa: F401

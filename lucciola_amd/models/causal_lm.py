@@ -23,6 +23,15 @@ from ..parts import BuildContext, ResidualStream, build_part
 from ..weights.loader import ParamDecl, WeightSource, load_declared, precision_notices
 
 
+def needs_of(part) -> tuple:
+    """A part's cache needs as a tuple: a part may state one need, several (pages and a piece of state, or the
+    needs of the parts it is made of), or none."""
+    need = part.cache_need()
+    if need is None:
+        return ()
+    return tuple(need) if isinstance(need, (tuple, list)) else (need,)
+
+
 class _LayerParts:
     """The parts of one layer, built from its spec, and the block that arranges them."""
 
@@ -183,7 +192,7 @@ class CausalLM:
             if entry.cache_of is not None or not caching:
                 needs.append(None)
             else:
-                mine = tuple(part.cache_need() for part in caching)
+                mine = tuple(need for part in caching for need in needs_of(part))
                 needs.append(mine[0] if len(mine) == 1 else mine)
         return needs
 

@@ -86,7 +86,8 @@ class Part:
         """What this part keeps in the cache: a ``cache.specs.CacheNeed`` (PagedKV, FixedState or
         a subclass of the part's own) or None.  What the need allocates is what the part finds
         as ``site.cache``; a paged need also finds ``site.pages`` (block table, slots, page
-        size)."""
+        size).  A part that keeps several things (pages and a piece of state per request) returns a
+        tuple of needs and finds the k-th as ``site.part(k)``."""
         return None
 
     def tables_epoch(self) -> int:

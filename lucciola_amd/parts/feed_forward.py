@@ -182,21 +182,37 @@ class RoutedGatedMLP(Part):
     (float32, plus a bias where ``router_bias``) pick the ``top`` largest; their weights are the
     softmax over the chosen logits alone.  ``shared_size`` > 0: a gated feed-forward of that inner
     size runs for every token and is added times sigmoid(w . x), one number per token (its
-    weight row rides along in the router's product).  The experts' products run over the (token,
-    choice) pairs sorted by expert, as for ``routed_mlp``; nothing passes the host."""
+    weight row rides along in the router's product; ``shared_gate`` False: it is added as it is).
+    ``scores`` "sigmoid": the scores are sigmoids of the logits, the ``top`` largest are chosen and weigh as
+    they are, not renormalised.  ``weigh`` "input": a chosen expert's weight multiplies what it reads, not what
+    it gives, expert(w x); both of its first products being linear, that is act(w gate x) * (w up x), formed
+    where the gated activation is.  The experts' products run over the (token, choice) pairs sorted by expert,
+    as for ``routed_mlp``; nothing passes the host."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int,
-                 activation: str = "silu", router_bias: bool = False, shared_size: int = 0):
+                 activation: str = "silu", router_bias: bool = False, shared_size: int = 0,
+                 scores: str = "softmax_chosen", weigh: str = "output", shared_gate: bool = True):
         super().__init__(hidden_size=hidden_size, intermediate_size=intermediate_size, experts=experts, top=top,
-                         activation=activation, router_bias=router_bias, shared_size=shared_size)
+                         activation=activation, router_bias=router_bias, shared_size=shared_size, scores=scores,
+                         weigh=weigh, shared_gate=shared_gate)
         if activation not in ops.GATE_ACTIVATIONS:
             raise ValueError(f"routed_gated_mlp: activation '{activation}' has no kernel")
         if not 1 <= int(top) <= int(experts):
             raise ValueError(f"routed_gated_mlp: top {top} of {experts} experts")
+        if scores not in ("softmax_chosen", "sigmoid"):
+            raise ValueError(f"routed_gated_mlp: scores '{scores}' have no kernel (softmax_chosen, sigmoid)")
+        if weigh not in ("output", "input"):
+            raise ValueError(f"routed_gated_mlp: weigh '{weigh}' is neither 'output' nor 'input'")
+        if scores == "sigmoid" and router_bias:
+            raise ValueError("routed_gated_mlp: sigmoid scores go without a router bias")
         self.H, self.I, self.E, self.top = int(hidden_size), int(intermediate_size), int(experts), int(top)
         self.activation, self.router_bias, self.S = activation, bool(router_bias), int(shared_size)
+        self.scores, self.weigh = scores, weigh
+        self.shared_gate = bool(shared_gate) and self.S > 0
+        if scores == "sigmoid" and self.shared_gate:
+            raise ValueError("routed_gated_mlp: with sigmoid scores the shared expert has no gate of its own")
         self.shared = (GatedMLP(hidden_size=self.H, intermediate_size=self.S, activation=activation)
                        if self.S else None)
 
@@ -210,13 +226,15 @@ class RoutedGatedMLP(Part):
             out[f"experts.{k}.down"] = ParamDecl((self.H, self.I))
         if self.shared is not None:
             out.update({"shared.gate": ParamDecl((self.S, self.H)), "shared.up": ParamDecl((self.S, self.H)),
-                        "shared.down": ParamDecl((self.H, self.S)), "shared_gate": ParamDecl((1, self.H))})
+                        "shared.down": ParamDecl((self.H, self.S))})
+            if self.shared_gate:
+                out["shared_gate"] = ParamDecl((1, self.H))
         return out
 
     def bind(self, tensors, ctx: BuildContext) -> None:
         self.dtype = ctx.dtype
         # one product gives the router's logits and, in its last column, the shared expert's gate
-        self.router = stack_rows([tensors["router"]] + ([tensors["shared_gate"]] if self.shared is not None else []))
+        self.router = stack_rows([tensors["router"]] + ([tensors["shared_gate"]] if self.shared_gate else []))
         self.bias = tensors["router_bias"].to(torch.float32).contiguous() if self.router_bias else None
         self.gate_up = stack_rows([t for k in range(self.E) for t in (tensors[f"experts.{k}.gate"],
                                                                        tensors[f"experts.{k}.up"])]
@@ -229,11 +247,21 @@ class RoutedGatedMLP(Part):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = ops.gemm(x, self.router, torch.float32)            # [T, E (+ 1)]
-        routing = ops.moe_route_logits(logits, self.E, self.top, self.bias, large_tiles=self.large_tiles)
+        if self.scores == "sigmoid":
+            routing = ops.moe_route_sigmoid(logits, self.top, large_tiles=self.large_tiles)
+        else:
+            routing = ops.moe_route_logits(logits, self.E, self.top, self.bias, large_tiles=self.large_tiles)
         both = ops.moe_experts(x, self.gate_up, routing, self.dtype, gather=True)
-        hidden = ops.gated_activation(both, self.activation)
+        if self.weigh == "input":
+            hidden = ops.gated_activation_weighted(both, self.activation, routing)
+        else:
+            hidden = ops.gated_activation(both, self.activation)
         y = ops.moe_experts(hidden, self.down, routing, torch.float32)
+        weighted = self.weigh == "output"
         if self.shared is None:
-            return ops.moe_combine(y, routing, self.dtype)
+            if weighted:
+                return ops.moe_combine(y, routing, self.dtype)
+            return ops.moe_combine_shared(y, routing, None, None, 0, self.dtype, weighted=False)
         extra = ops.value(self.shared.forward(x))
-        return ops.moe_combine_shared(y, routing, extra, logits, self.E, self.dtype)
+        return ops.moe_combine_shared(y, routing, extra, logits if self.shared_gate else None, self.E, self.dtype,
+                                      weighted=weighted)

@@ -100,31 +100,39 @@ class LayerNorm(Part):
     """``y = (x - mean) / sqrt(var + eps) * w + b`` over the last dimension, the variance being
     the mean of the squared deviations; float32 arithmetic.  Where the branch output that waits
     to be added is itself to be normed first (``ops.NormedBranch``: a block with a norm behind
-    each branch), one kernel norms the branch, adds it to the stream and norms the stream."""
+    each branch), one kernel norms the branch, adds it to the stream and norms the stream.  ``bias``
+    False: the norm has a weight only.  ``branch_scale``: the branch output that waits is multiplied by
+    this number as it is added to the stream (a model whose layers are x + m branch(norm(x)))."""
 
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
-        super().__init__(size=size, eps=eps)
+    def __init__(self, size: int, eps: float, bias: bool = True, branch_scale: float = 1.0):
+        super().__init__(size=size, eps=eps, bias=bias, branch_scale=branch_scale)
         self.size, self.eps = int(size), float(eps)
+        self.has_bias, self.branch_scale = bool(bias), float(branch_scale)
         self.weight = self.bias = None
         self.dtype = None
 
     def declare(self) -> Dict[str, ParamDecl]:
-        return {"weight": ParamDecl((self.size,), role="vector", init="ones_plus_normal"),
-                "bias": ParamDecl((self.size,), role="vector", init="normal")}
+        out = {"weight": ParamDecl((self.size,), role="vector", init="ones_plus_normal")}
+        if self.has_bias:
+            out["bias"] = ParamDecl((self.size,), role="vector", init="normal")
+        return out
 
     def bind(self, tensors, ctx: BuildContext) -> None:
-        self.weight, self.bias = tensors["weight"], tensors["bias"]
+        self.weight = tensors["weight"]
+        self.bias = tensors["bias"] if self.has_bias else torch.zeros_like(self.weight)
         self.dtype = ctx.dtype
 
     def add_norm(self, stream: ResidualStream, scaled: bool = False):
-        x = ops.layer_norm(stream.h, stream.pending, self.weight, self.bias, self.eps, self.dtype)
+        x = ops.layer_norm(stream.h, stream.pending, self.weight, self.bias, self.eps, self.dtype,
+                           branch_scale=self.branch_scale)
         stream.pending = None
         return x
 
     def add_norm_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
-        return ops.layer_norm(stream.h, stream.pending, self.weight, self.bias, self.eps, self.dtype, rows=rows)
+        return ops.layer_norm(stream.h, stream.pending, self.weight, self.bias, self.eps, self.dtype, rows=rows,
+                              branch_scale=self.branch_scale)
 
     def behind(self, branch) -> "ops.NormedBranch":
         """``branch`` (a branch's output) as something that is normed by this norm before it is

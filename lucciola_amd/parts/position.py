@@ -12,7 +12,10 @@ the same, the kernels that rotate differ) and a stretching of the frequencies fo
 longer than the one trained on (``scaling``, the YaRN rule: with dim(t) = rot ln(original /
 (2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot - 1) and
 ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), frequency i becomes f_i / factor * ramp_i +
-f_i (1 - ramp_i), and cosines and sines are multiplied by 0.1 ln(factor) + 1).
+f_i (1 - ramp_i), and cosines and sines are multiplied by 0.1 ln(factor) + 1).  A ``scaling`` with
+``kind`` "wavelength" goes by each frequency's wavelength l = 2 pi / f against the ``original`` context:
+f is kept where l < original / high, divided by ``factor`` where l > original / low, and between the two,
+with s = (original / l - low) / (high - low), it becomes (1 - s) f / factor + s f; nothing else changes.
 """
 from __future__ import annotations
 
@@ -47,8 +50,15 @@ class Rotary(Part):
             raise ValueError(f"rotary: pairing '{pairing}' is neither 'half' nor 'interleaved'")
         self.rotary_dim, self.theta, self.pairing = int(rotary_dim), float(theta), pairing
         self.scaling = None
-        if scaling:
+        self.scaling_kind = str(scaling.get("kind", "yarn")) if scaling else None
+        if scaling and self.scaling_kind == "wavelength":
+            self.scaling = ("wavelength",) + tuple(float(scaling[k]) for k in ("factor", "original", "low", "high"))
+            if self.scaling[1] <= 0 or self.scaling[2] <= 0 or self.scaling[4] <= self.scaling[3]:
+                raise ValueError("rotary: wavelength scaling needs factor > 0, original > 0 and high > low")
+        elif scaling and self.scaling_kind == "yarn":
             self.scaling = tuple(float(scaling[k]) for k in ("factor", "original", "fast", "slow"))
+        elif scaling:
+            raise ValueError(f"rotary: scaling kind '{self.scaling_kind}' is neither 'yarn' nor 'wavelength'")
         self.initial = int(max_positions)
         self._shared = _SharedTable()
         self._device = None
@@ -74,7 +84,14 @@ class Rotary(Part):
         inv_freq = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64),
                                    2.0 * i / self.rotary_dim)
         magnitude = 1.0
-        if self.scaling is not None:
+        if self.scaling is not None and self.scaling[0] == "wavelength":
+            _, factor, original, low, high = self.scaling
+            wavelength = 2.0 * math.pi / inv_freq
+            blend = (original / wavelength - low) / (high - low)
+            between = (1.0 - blend) * inv_freq / factor + blend * inv_freq
+            inv_freq = torch.where(wavelength < original / high, inv_freq,
+                                   torch.where(wavelength > original / low, inv_freq / factor, between))
+        elif self.scaling is not None:
             factor, original, fast, slow = self.scaling
 
             def turn_dim(turns: float) -> float:

@@ -361,7 +361,7 @@ def layer_norm_act(x, weight, bias, eps):
     return _layer_norm64(x.to(F64), weight, bias, eps).to(x.dtype)
 
 
-def layer_norm(h, delta, weight, bias, eps, out_dtype, rows=None):
+def layer_norm(h, delta, weight, bias, eps, out_dtype, rows=None, branch_scale=1.0):
     from lucciola_amd.kernels import ops
     if isinstance(delta, ops.NormedBranch):
         delta = _layer_norm64(delta.x.to(F64), delta.weight, delta.bias, delta.eps).to(torch.float32)
@@ -369,12 +369,12 @@ def layer_norm(h, delta, weight, bias, eps, out_dtype, rows=None):
         delta = delta.value()
     if rows is None:
         if delta is not None:
-            h += delta.to(torch.float32)
+            h += (branch_scale * delta.to(F64)).to(torch.float32)
         v = h.to(F64)
     else:
         v = h[rows.long()].to(F64)
         if delta is not None:
-            v = (h[rows.long()] + delta[rows.long()].to(torch.float32)).to(F64)
+            v = (h[rows.long()] + (branch_scale * delta[rows.long()].to(F64)).to(torch.float32)).to(F64)
     return _layer_norm64(v, weight, bias, eps).to(out_dtype)
 
 
@@ -532,10 +532,129 @@ def moe_route_logits(logits, experts, top, bias=None, large_tiles=False):
     return r
 
 
-def moe_combine_shared(y, routing, shared, gates, gate_column, out_dtype):
+def moe_combine_shared(y, routing, shared, gates, gate_column, out_dtype, weighted=True):
     T, top = routing.ids.shape
-    total = (y.to(F64).view(T, top, -1) * routing.weights.to(F64)[:, :, None]).sum(1)
-    return (total + torch.sigmoid(gates[:, gate_column].to(F64))[:, None] * shared.to(F64)).to(out_dtype)
+    total = y.to(F64).view(T, top, -1)
+    if weighted:
+        total = total * routing.weights.to(F64)[:, :, None]
+    total = total.sum(1)
+    if shared is not None:
+        gate = torch.sigmoid(gates[:, gate_column].to(F64))[:, None] if gates is not None else 1.0
+        total = total + gate * shared.to(F64)
+    return total.to(out_dtype)
+
+
+def gated_activation_weighted(gu, kind, routing):
+    """Rows in (token, choice) order, as :func:`moe_experts` leaves them here."""
+    I = gu.shape[1] // 2
+    w = routing.weights.to(F64).reshape(-1, 1)
+    g, u = w * gu[:, :I].to(F64), w * gu[:, I:].to(F64)
+    a = g / (1 + torch.exp(-g)) if kind == "silu" else _act(g, kind)
+    return (a * u).to(gu.dtype)
+
+
+MASKED_ATTENTION_MAX = 256
+SHORT_CONV_MAX_TAPS = 8
+
+
+def _convolved(proj, C, taps, tail, tok_req, q_offsets, slot_ids, bias=None):
+    """The first C columns of proj through their causal convolutions, float64 [T, C]."""
+    K = taps.shape[1]
+    x = _conv_inputs(proj, tail, C, K, tok_req, q_offsets, slot_ids)
+    y = torch.zeros(proj.shape[0], C, dtype=F64)
+    for j in range(K):
+        y += x[j] * taps.to(F64)[:, K - 1 - j][None, :]
+    return y if bias is None else y + bias.to(F64)
+
+
+def attention_prepare(proj, nq, nk, nv, d, dv, out_dtype, k_cache, v_cache, rows, taps=None, tail=None, tok_req=None,
+                      q_offsets=None, slot_ids=None, table=None, rot=0, positions=None, unit_eps=None):
+    T = proj.shape[0]
+    C = (nq + nk) * d + nv * dv
+    y = proj[:, :C].to(F64) if taps is None else _convolved(proj, C, taps, tail, tok_req, q_offsets, slot_ids)
+    qk = y[:, :(nq + nk) * d].reshape(T, nq + nk, d).clone()
+    if table is not None:
+        cs = table[positions.long()].to(F64)
+        cos, sin = cs[:, None, :rot // 2], cs[:, None, rot // 2:]
+        a, b = qk[..., 0:rot:2].clone(), qk[..., 1:rot:2].clone()
+        qk[..., 0:rot:2] = a * cos - b * sin
+        qk[..., 1:rot:2] = b * cos + a * sin
+    if unit_eps is not None:
+        qk = qk / torch.sqrt((qk * qk).mean(-1, keepdim=True) + unit_eps)
+    if rows is not None:
+        keep = rows >= 0
+        k_cache[rows[keep].long()] = qk[keep, nq:].reshape(-1, nk * d).to(k_cache.dtype)
+        v_cache[rows[keep].long()] = y[keep, (nq + nk) * d:].to(v_cache.dtype)
+    return qk[:, :nq].reshape(T, nq * d).to(out_dtype)
+
+
+def masked_attention(q, k_cache, v_cache, tok_req, positions, block_table, page_size, heads, kv_heads, maps, d, dv,
+                     scale, chunk=0, window=0, r1=None, r2=None, sink=None, subtract=0.0, unit_eps=None,
+                     out_scale=1.0, gate=None, gate_column=0):
+    T = q.shape[0]
+    kc = k_cache.reshape(-1, kv_heads, maps, d).to(F64)
+    vc = v_cache.reshape(-1, kv_heads, dv).to(F64)
+    qq = q.to(F64).view(T, heads, maps, d)
+    out = torch.zeros(T, heads, dv, dtype=F64)
+    for t in range(T):
+        p, r = int(positions[t]), int(tok_req[t])
+        lo = 0
+        if chunk > 0:
+            lo = p - p % chunk
+        if window > 0:
+            lo = max(lo, p - window + 1)
+        js = torch.arange(lo, p + 1)
+        rows = block_table[r].long()[js // page_size] * page_size + js % page_size
+        for h in range(heads):
+            g = h // (heads // kv_heads)
+            a = []
+            for m in range(maps):
+                s = (kc[rows, g, m] @ qq[t, h, m]) * scale
+                if r1 is not None:
+                    s = s - float(r1[h]) * torch.log1p(float(r2[h]) * (p - js).to(F64))
+                top = s.max() if sink is None else torch.maximum(s.max(), sink[h].to(F64))
+                e = torch.exp(s - top)
+                total = e.sum() + (torch.exp(sink[h].to(F64) - top) if sink is not None else 0.0)
+                a.append((e / total) @ vc[rows, g])
+            o = a[0] if maps == 1 else a[0] - subtract * a[1]
+            if unit_eps is not None:
+                o = o / torch.sqrt((o * o).mean() + unit_eps) * out_scale
+            out[t, h] = o
+    out = out.view(T, heads * dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate[:, gate_column:gate_column + heads * dv].to(F64))
+    return out.to(q.dtype)
+
+
+def state_space_prepare(proj, heads, groups, state, value_dim, taps, bias, tail, dt_bias, a_log, tok_req, q_offsets,
+                        slot_ids):
+    T = proj.shape[0]
+    inner = heads * value_dim
+    C = inner + 2 * groups * state
+    y = _convolved(proj, C, taps, tail, tok_req, q_offsets, slot_ids, bias)
+    y = y * torch.sigmoid(y)
+    rep = heads // groups
+    B = y[:, inner:inner + groups * state].view(T, groups, state).repeat_interleave(rep, dim=1)
+    Cm = y[:, inner + groups * state:].view(T, groups, state).repeat_interleave(rep, dim=1)
+    step = torch.nn.functional.softplus(proj[:, C + inner:].to(F64) + dt_bias.to(F64))        # [T, heads]
+    decay = torch.exp(-torch.exp(a_log.to(F64)) * step)
+    coef = torch.stack([decay[:, :, None].expand(T, heads, state), step[:, :, None] * B, Cm])
+    return coef.reshape(3, T, heads * state).to(torch.float32).contiguous(), y[:, :inner].to(torch.float32).contiguous()
+
+
+def state_space_readout(o, x, gates, z_column, skip, heads, value_dim, weight, parts, eps, out_dtype):
+    T, n = o.shape
+    z = gates[:, z_column:z_column + n].to(F64)
+    y = (o.to(F64) + skip.to(F64).repeat_interleave(value_dim)[None, :] * x.to(F64)) * (z * torch.sigmoid(z))
+    y = y.view(T, parts, n // parts)
+    y = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps)
+    return (y.reshape(T, n) * weight.to(F64)).to(out_dtype)
+
+
+def scaled_sum(a, a_scale, b, b_scale):
+    a = a if isinstance(a, torch.Tensor) else a.value()
+    b = b if isinstance(b, torch.Tensor) else b.value()
+    return (a_scale * a.to(F64) + b_scale * b.to(F64)).to(torch.float32)
 
 
 def moe_large_tiles(x_dtype, up, down):
@@ -547,7 +666,9 @@ ALL = ("layer_norm", "layer_norm_act", "embedding_sinusoid", "gated_activation",
        "head_gate_norm", "moe_route_logits", "moe_combine_shared", "feed_tokens", "attention_takes_shares", "embedding", "rmsnorm", "rmsnorm_act", "gemm", "qk_norm_rope_write", "attention",
        "swiglu", "sample", "dynamic_tanh", "stream_add", "activation", "gemm_act", "grouped_gemm",
        "latent_prepare", "latent_attention", "moe_route", "moe_experts", "moe_combine",
-       "scale_", "token_shift", "rms_shift", "moe_route_sigmoid", "lightning_prepare", "lightning_readout")
+       "scale_", "token_shift", "rms_shift", "moe_route_sigmoid", "lightning_prepare", "lightning_readout",
+       "gated_activation_weighted", "attention_prepare", "masked_attention", "state_space_prepare",
+       "state_space_readout", "scaled_sum")
 
 
 def install(monkeypatch):
