@@ -77,9 +77,9 @@ def rotate_interleaved(x, positions, freqs):
 def differential_attention(h, w: Dict[str, torch.Tensor], p: str, m: dict, eps: float):
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = causal_conv(h @ w[p + "q"].T, w[p + "q.conv"])
-    k = causal_conv(h @ w[p + "k"].T, w[p + "k.conv"])
-    v = causal_conv(h @ w[p + "v"].T, w[p + "v.conv"])
+    q, k, v = h @ w[p + "q"].T, h @ w[p + "k"].T, h @ w[p + "v"].T
+    if m.get("conv"):
+        q, k, v = (causal_conv(u, w[p + name + ".conv"]) for u, name in ((q, "q"), (k, "k"), (v, "v")))
     q = q.view(T, H * 2, d)
     k = k.view(T, G * 2, d)
     v = v.view(T, G, dv)
@@ -186,8 +186,8 @@ def routed_experts(h, w, p: str, mlp: dict):
 def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], keep_layers: bool = False):
     """Logits [T, vocab] of one sequence; with ``keep_layers`` also the stream after every layer."""
     eps = cfg["norm"]["eps"]
-    mult = cfg["residual_mult"]
-    x = w["embed"][torch.tensor(tokens)] * cfg["embedding"]["scale"]
+    mult = cfg.get("residual_mult", 1.0)
+    x = w["embed"][torch.tensor(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
     after = []
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
@@ -202,5 +202,5 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], keep_layer
             h = layer_norm(x, w[p + "norm2"], eps)
             x = x + mult * routed_experts(h, w, p + "mlp.", layer["mlp"])
         after.append(x)
-    logits = layer_norm(x, w["final.norm"], eps) @ w["head"].T * cfg["logit_scale"]
+    logits = layer_norm(x, w["final.norm"], eps) @ w["head"].T * cfg.get("logit_scale", 1.0)
     return (logits, after) if keep_layers else logits
