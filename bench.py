@@ -408,6 +408,32 @@ def kikunex_design_config(name, routed=True):
             "logit_scale": 0.5, "initializer_range": 0.02, "layers": layers}
 
 
+def rununex_design_config(name, routed=True):
+    """The Rununex decoder at the same width, heads, head size, feed-forward width, vocabulary and depth:
+    differential attention (two maps of 64 query/key entries a head, values of 128, four taps on q, k and v, all
+    entries rotated, chunks of 4,096) and the two mixers side by side in turn (attention with unit q and k, a
+    distance bias, a sink and a gate, heads of 128, chunks of 4,096, beside a state-space mixer of width / 64
+    heads of 64 with a state of 128 in 8 groups); every layer has routed gated experts fed their weighted input
+    (4 of 32 experts of ff / 4 and a shared one of ff / 4; ``routed`` False: one expert of ff / 2 that every token
+    takes and a shared one of ff / 2, which move a dense layer's weights)."""
+    width, heads, ff = DESIGN_SIZES[name]
+    kv = max(1, heads // 4)
+    attention = {"heads": heads, "kv_heads": kv, "dim": 64, "vdim": 128, "scale": 64 ** -0.5, "diff": 0.3, "conv": 4,
+                 "mask": {"size": 4096},
+                 "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    left = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 0.125, "mask": {"size": 4096}}
+    right = {"heads": width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
+    both = {"left": left, "right": right, "left_scale": 0.8, "right_scale": 1.1}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}, "shared": {"ff": ff // 4}}
+    if not routed:
+        moe = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 1, "top": 1}, "shared": {"ff": ff // 2}}
+    layers = [{"type": "attention", "mixer": attention, "mlp": moe}, {"type": "parallel", "mixer": both, "mlp": moe},
+              {"type": "attention", "mixer": attention, "mlp": moe}, {"type": "parallel", "mixer": both, "mlp": moe}]
+    return {"architecture": "Rununex", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": float(width) ** 0.5}, "residual_mult": 0.7, "logit_scale": 0.25,
+            "initializer_range": 0.02, "layers": layers}
+
+
 def design_run(cfg, dtype, dev, block_size, prompt, batches, context, steps):
     """Prompt and decode throughput of one configuration through the runner's own step."""
     import torch
@@ -490,10 +516,10 @@ def designs_workload(args, dev):
                 results[key] = design_run(pubodra, dtype, dev, args.block_size, args.prefill_tokens, batches,
                                           args.design_context, args.steps)
                 say(f"{key}: {results[key]}")
-        for model in ("larupel", "larupel_dense", "kikunex", "kikunex_dense"):
+        for model in ("larupel", "larupel_dense", "kikunex", "kikunex_dense", "rununex", "rununex_dense"):
             if model in wanted:
                 key = f"{name}/{model}"
-                make = larupel_design_config if model.startswith("larupel") else kikunex_design_config
+                make = {"l": larupel_design_config, "k": kikunex_design_config, "r": rununex_design_config}[model[0]]
                 results[key] = design_run(make(name, routed="dense" not in model), dtype, dev,
                                           args.block_size, args.prefill_tokens, batches, args.design_context, args.steps)
                 say(f"{key}: {results[key]}")
@@ -544,7 +570,8 @@ def main() -> int:
     ap.add_argument("--design-sizes", default="w2048,w4096", help="designs: which of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-batches", default="8,64", help="designs: decode batch sizes")
     ap.add_argument("--design-models", default="qwen3,pubodra_dense,pubodra_routed,larupel",
-                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel, larupel_dense, kikunex, kikunex_dense")
+                    help="designs: which of qwen3, pubodra_dense, pubodra_routed, larupel, larupel_dense, kikunex, kikunex_dense, "
+                         "rununex, rununex_dense")
     ap.add_argument("--design-context", type=int, default=2048, help="designs: tokens a decoding request holds")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "designs"],
                     help="decode: the default line; mixed: only the 0.6B-shaped mixed workload, as a line of its own")

@@ -126,7 +126,8 @@ class PagedRows(CacheNeed):
     value heads of different numbers or sizes, several key maps that share a value).  ``window`` as for
     :class:`PagedKV`.
 
-    Memory per site, token-major: keys ``[pages, page, key_width]``, values ``[pages, page, value_width]``; any
+    Memory per site: keys token-major ``[pages, page, key_width]``, values transposed inside a page ``[pages,
+    value_width, page]`` (a matrix-core operand wants a value entry's neighbouring positions side by side); any
     page size."""
 
     key_width: int
@@ -141,7 +142,7 @@ class PagedRows(CacheNeed):
     def allocate(self, layout: CacheLayout, dtype: torch.dtype, device):
         pages, page = layout.kernel_pages, layout.kernel_page
         return (torch.zeros((pages, page, self.key_width), dtype=dtype, device=device),
-                torch.zeros((pages, page, self.value_width), dtype=dtype, device=device))
+                torch.zeros((pages, self.value_width, page), dtype=dtype, device=device))
 
 
 @dataclass(frozen=True)

@@ -9,8 +9,9 @@
 //   a_m = sum_j exp(s_j) v_g,j / (sum_j exp(s_j) + exp(sink_h))              (the sink where it is given)
 //   maps = 1: o = a_0;   maps = 2: o = a_0 - lambda a_1
 //   unit_out: o <- o / sqrt(mean(o^2) + eps) * out_scale;   gate: o <- o sigmoid(gate_(h, .))
-// Cache layouts, token-major: keys [pages * page, kv_heads * maps * d], values [pages * page, kv_heads * dv];
-// the entry of position j of request r lies at row block_table[r][j / page] * page + j % page.
+// Cache layouts: keys token-major, [pages, page, kv_heads * maps * d]; values transposed inside a page, [pages,
+// kv_heads * dv, page] (the matrix-core kernel's operand wants a value entry's neighbouring keys side by side).
+// Position j of request r lies in page block_table[r][j / page] at place j % page.
 //
 // The keys are walked in tiles of 256 from lo on, with a running maximum and sum per map: the order of
 // every addition is a function of the query's position alone, so a token's result has the same bits in
@@ -104,8 +105,8 @@ __global__ __launch_bounds__(MA_THREADS) void masked_attention_kernel(
         if (active)
             for (int jj = grp; jj < count; jj += groups) {
                 const int j = c0 + jj;
-                const size_t row = (size_t)table[j / page_size] * page_size + j % page_size;
-                const float v = to_f32(v_cache[row * v_row + (size_t)g * dv + dim]);
+                const float v = to_f32(v_cache[((size_t)table[j / page_size] * v_row + (size_t)g * dv + dim) * page_size
+                                               + j % page_size]);
 #pragma unroll
                 for (int m = 0; m < MAPS; ++m) acc[m] = fmaf(ps[m][jj], v, acc[m]);
             }
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(MA_THREADS) void attention_prepare_kernel(
     const float* __restrict__ taps, int K, const float* __restrict__ tails, const int* __restrict__ tok_req,
     const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, const float* __restrict__ table, int rot,
     const int* __restrict__ positions, int unit, float eps, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, const int* __restrict__ rows) {
+    T* __restrict__ v_cache, const int* __restrict__ rows, int page_size) {
     const int t = blockIdx.x, lane = threadIdx.x & (kWave - 1);
     const int u = blockIdx.y * (MA_THREADS / kWave) + threadIdx.x / kWave;
     if (u >= nq + nk + nv) return;
@@ -191,19 +192,25 @@ __global__ __launch_bounds__(MA_THREADS) void attention_prepare_kernel(
     float inv = 1.f;
     if (unit && !is_v) inv = 1.f / sqrtf(wave_sum(ss) / (float)width + eps);
     T* dst;
+    size_t step = 1;                // between neighbouring entries of the head
     if (u < nq) {
         dst = q_out + (size_t)t * nq * d + (size_t)u * d;
     } else {
         if (!rows || rows[t] < 0) return;
-        dst = is_v ? v_cache + (size_t)rows[t] * nv * dv + (size_t)(u - nq - nk) * dv
-                   : k_cache + (size_t)rows[t] * nk * d + (size_t)(u - nq) * d;
+        if (is_v) {                 // values lie transposed inside their page: [entry][place]
+            dst = v_cache + ((size_t)(rows[t] / page_size) * nv * dv + (size_t)(u - nq - nk) * dv) * page_size
+                  + rows[t] % page_size;
+            step = page_size;
+        } else {
+            dst = k_cache + (size_t)rows[t] * nk * d + (size_t)(u - nq) * d;
+        }
     }
 #pragma unroll
     for (int k = 0; k < 2; ++k)
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int at = 2 * (lane + kWave * k) + e;
-            if (at < width) dst[at] = from_f32<T>(x[k][e] * inv);
+            if (at < width) dst[at * step] = from_f32<T>(x[k][e] * inv);
         }
 }
 
@@ -249,7 +256,7 @@ LC_API int lc_attention_prepare(const float* proj, int cols, int T, int nq, int 
                                 const float* taps, int K, const float* tails, const int* tok_req,
                                 const int* q_offsets, const int* slot_ids, const float* table, int rot,
                                 const int* positions, int unit, float eps, void* q_out, void* k_cache, void* v_cache,
-                                int dt, const int* rows, hipStream_t stream) {
+                                int dt, const int* rows, int page_size, hipStream_t stream) {
     LC_CHECK(T >= 0 && nq > 0 && nk >= 0 && nv >= 0 && d > 0 && dv > 0 && cols >= (nq + nk) * d + nv * dv,
              "attention prepare: bad sizes");
     LC_CHECK(d <= MA_MAX && dv <= MA_MAX, "attention prepare: heads of %d/%d entries are above %d", d, dv, MA_MAX);
@@ -258,17 +265,17 @@ LC_API int lc_attention_prepare(const float* proj, int cols, int T, int nq, int 
     LC_CHECK(!taps || (K >= 1 && K <= SHORT_CONV_MAX_TAPS && tok_req && q_offsets && slot_ids && (K == 1 || tails)),
              "attention prepare: a convolution needs 1 to %d taps, the tails and the request lists", SHORT_CONV_MAX_TAPS);
     LC_CHECK(!table || (rot > 0 && rot % 2 == 0 && rot <= d && positions), "attention prepare: bad rotation");
-    LC_CHECK(!rows || (k_cache && v_cache), "attention prepare: rows without a cache");
+    LC_CHECK(!rows || (k_cache && v_cache && page_size > 0), "attention prepare: rows without a cache");
     const int units = nq + nk + nv, per = MA_THREADS / kWave;
     const dim3 grid(T, (units + per - 1) / per);
     if (dt == DT_F32)
         attention_prepare_kernel<float><<<grid, MA_THREADS, 0, stream>>>(
             proj, cols, T, nq, nk, nv, d, dv, taps, K, tails, tok_req, q_offsets, slot_ids, table, rot, positions, unit,
-            eps, (float*)q_out, (float*)k_cache, (float*)v_cache, rows);
+            eps, (float*)q_out, (float*)k_cache, (float*)v_cache, rows, page_size);
     else if (dt == DT_BF16)
         attention_prepare_kernel<bf16><<<grid, MA_THREADS, 0, stream>>>(
             proj, cols, T, nq, nk, nv, d, dv, taps, K, tails, tok_req, q_offsets, slot_ids, table, rot, positions, unit,
-            eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, rows);
+            eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, rows, page_size);
     else
         LC_CHECK(false, "attention prepare: unknown dtype %d", dt);
     LC_LAUNCH_CHECK("attention_prepare");

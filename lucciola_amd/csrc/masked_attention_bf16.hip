@@ -1,0 +1,350 @@
+// The masked attention of masked_attention.hip on the matrix cores, for bfloat16 caches whose sizes fit:
+// key heads of a multiple of 8 entries up to 128, value heads of a multiple of 16 up to 128, pages of a
+// multiple of 16 tokens.  Same formulas, same cache (keys token-major, values transposed inside a page);
+// scores, softmax, sink, bias and the heads' combination are float32, the two products take bfloat16
+// operands: the weights go into P.V as two bfloat16 numbers each (the rounded weight and the rounding's
+// remainder, two products), so that they count with 16 bits of mantissa and not with 8.
+//
+// Work comes as the step's tiles (first token row, tokens, request, first position: up to 16 tokens of one
+// request); a workgroup of eight waves serves a tile and one kv head.
+//   A tile of several tokens: a wave's 16 columns are the tile's tokens for one query head of the kv head's
+//   group; where the group has fewer than eight heads, the waves of a head share out the blocks of keys.
+//   A lone token: the 16 columns are query heads of the group, and all eight waves share out the blocks.
+// Waves that shared a column's keys leave their maxima, sums and rows in LDS, and the first of them takes the
+// others in, in their order.  A wave asks for the next block's keys before it works on this one's.
+// Keys are walked in blocks of 16 (one part of a page).  S^T = K Q^T (16x16x32: a lane's operand is 16 bytes
+// in a row of a key, straight from memory) leaves a lane with four keys of one query column, which is the
+// operand P^T of O^T += V^T P^T (16x16x16; V^T's operand is four neighbouring keys of one value entry, 8
+// bytes in a row of the transposed page), so the weights never leave the registers.
+#include "common.h"
+
+namespace lc {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int MB_WAVES = 8;
+constexpr int MB_THREADS = MB_WAVES * kWave;
+
+struct MaskedArgs {
+    const bf16* q;
+    const bf16* k_cache;
+    const bf16* v_cache;
+    const int* tiles;
+    const int* block_table;
+    int max_blocks, page_size, heads, kv_heads, d, dv;
+    float scale;
+    int chunk, window;
+    const float* r1;
+    const float* r2;
+    const float* sink;
+    float lambda;
+    int unit_out;
+    float eps, out_scale;
+    const float* gate;
+    int gate_stride, gate_column;
+    bf16* out;
+};
+
+__device__ __forceinline__ short bits_of(__bf16 v) { return __builtin_bit_cast(short, v); }
+
+// over the four lanes that hold one query column (lane, lane ^ 16, lane ^ 32, lane ^ 48)
+__device__ __forceinline__ float column_max4(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, kWave));
+    return fmaxf(v, __shfl_xor(v, 32, kWave));
+}
+__device__ __forceinline__ float column_sum4(float v) {
+    v += __shfl_xor(v, 16, kWave);
+    return v + __shfl_xor(v, 32, kWave);
+}
+
+template <int DVB, int MAPS>
+struct ColumnState {
+    float m[MAPS], l[MAPS];
+    floatx4 o[MAPS][DVB];       // O^T: value entries 16 t + 4 (lane / 16) + i of the lane's query column
+};
+
+// The lane's column: token row `tok`, head `head`, position `pos` (-1: no such column), first visible key `lo`.
+// Blocks first, first + stride, ... <= last of 16 keys each.
+template <int DSTEPS, int DVB, int MAPS>
+__device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const MaskedArgs& a, int g, int tok, int head,
+                                              int pos, int lo, const int* __restrict__ table, int first, int last,
+                                              int stride, int lane) {
+    const int quad = lane >> 4, col = lane & 15;
+    const size_t k_row = (size_t)a.kv_heads * MAPS * a.d;
+    bf16x8 bq[MAPS][DSTEPS];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+        for (int s = 0; s < DSTEPS; ++s) {
+            const int e = s * 32 + quad * 8;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) bq[m][s][x] = (__bf16)0.f;
+            if (pos >= 0 && e < a.d)
+                bq[m][s] = *reinterpret_cast<const bf16x8*>(a.q + ((size_t)tok * a.heads + head) * MAPS * a.d + m * a.d + e);
+        }
+    const float bias1 = (a.r1 && pos >= 0) ? a.r1[head] : 0.f, bias2 = (a.r1 && pos >= 0) ? a.r2[head] : 0.f;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+        st.m[m] = -INFINITY;
+        st.l[m] = 0.f;
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) st.o[m][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    auto load_keys = [&](bf16x8 (&dst)[MAPS][DSTEPS], int b) {
+        const int key0 = b * 16;
+        const size_t row0 = (size_t)table[key0 / a.page_size] * a.page_size + key0 % a.page_size;
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+            for (int s = 0; s < DSTEPS; ++s) {
+                const int e = s * 32 + quad * 8;
+#pragma unroll
+                for (int x = 0; x < 8; ++x) dst[m][s][x] = (__bf16)0.f;
+                if (e < a.d)
+                    dst[m][s] = *reinterpret_cast<const bf16x8*>(a.k_cache + (row0 + col) * k_row + ((size_t)g * MAPS + m) * a.d + e);
+            }
+    };
+    auto load_values = [&](short4v (&dst)[DVB], int b) {
+        const int key0 = b * 16;
+        const int page = table[key0 / a.page_size], within = key0 % a.page_size;
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) {
+            dst[t] = short4v{0, 0, 0, 0};
+            if (t * 16 < a.dv)
+                dst[t] = *reinterpret_cast<const short4v*>(
+                    a.v_cache + ((size_t)page * a.kv_heads * a.dv + (size_t)g * a.dv + t * 16 + col) * a.page_size + within + quad * 4);
+        }
+    };
+    // the next block's values travel ahead as well where the registers hold them
+    constexpr bool VALUES_AHEAD = DSTEPS * MAPS * 4 + DVB * MAPS * 4 + DVB * 4 <= 120;
+    bf16x8 ka[MAPS][DSTEPS], kn[MAPS][DSTEPS];
+    short4v va[DVB], vn[DVB];
+    if (first <= last) {
+        load_keys(ka, first);
+        if constexpr (VALUES_AHEAD) load_values(va, first);
+    }
+    for (int b = first; b <= last; b += stride) {
+        const int key0 = b * 16;
+        if constexpr (!VALUES_AHEAD) load_values(va, b);
+        if (b + stride <= last) {           // on their way while this block is worked on
+            load_keys(kn, b + stride);
+            if constexpr (VALUES_AHEAD) load_values(vn, b + stride);
+        }
+        const int j0 = key0 + quad * 4;
+        float far[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) far[v] = a.r1 ? bias1 * __logf(1.f + bias2 * (float)max(pos - (j0 + v), 0)) : 0.f;
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) {
+            floatx4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < DSTEPS; ++i) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[m][i], bq[m][i], s, 0, 0, 0);
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int j = j0 + v;
+                s[v] = (j >= lo && j <= pos) ? fmaf(s[v], a.scale, -far[v]) : -INFINITY;
+                mx = fmaxf(mx, s[v]);
+            }
+            mx = column_max4(mx);
+            const float m_new = fmaxf(st.m[m], mx);
+            const float base = m_new == -INFINITY ? 0.f : m_new;      // a column that has seen no key yet
+            const float alpha = __expf(st.m[m] - base);
+            float p[4], psum = 0.f;
+            short4v hi, lw;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                p[v] = __expf(s[v] - base);
+                psum += p[v];
+                const __bf16 top = (__bf16)p[v];
+                hi[v] = bits_of(top);
+                lw[v] = bits_of((__bf16)(p[v] - (float)top));
+            }
+            st.l[m] = fmaf(st.l[m], alpha, column_sum4(psum));
+            st.m[m] = m_new;
+#pragma unroll
+            for (int t = 0; t < DVB; ++t) {
+                st.o[m][t] *= alpha;
+                st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], hi, st.o[m][t], 0, 0, 0);
+                st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], lw, st.o[m][t], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+            for (int i = 0; i < DSTEPS; ++i) ka[m][i] = kn[m][i];
+        if constexpr (VALUES_AHEAD)
+#pragma unroll
+            for (int t = 0; t < DVB; ++t) va[t] = vn[t];
+    }
+}
+
+// The lane's column is done: sink, the maps' combination, the unit norm, the gate; four entries a block written.
+template <int DVB, int MAPS>
+__device__ __forceinline__ void finish_column(const ColumnState<DVB, MAPS>& st, const MaskedArgs& a, int tok, int head,
+                                              int pos, int lane) {
+    const int quad = lane >> 4;
+    floatx4 o[DVB];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+        float top = st.m[m], sunk = 0.f;
+        if (a.sink && pos >= 0) {
+            top = fmaxf(st.m[m], a.sink[head]);
+            sunk = expf(a.sink[head] - top);
+        }
+        const float shrink = pos >= 0 ? expf(st.m[m] - top) : 0.f;
+        const float denom = fmaf(st.l[m], shrink, sunk);
+        const float w = denom > 0.f ? shrink / denom : 0.f;
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) {
+            if (m == 0) o[t] = st.o[0][t] * w;
+            else o[t] -= st.o[m][t] * (w * a.lambda);
+        }
+    }
+    if (a.unit_out) {
+        float ss = 0.f;
+#pragma unroll
+        for (int t = 0; t < DVB; ++t)
+            if (t * 16 < a.dv)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ss = fmaf(o[t][i], o[t][i], ss);
+        const float inv = a.out_scale / sqrtf(column_sum4(ss) / (float)a.dv + a.eps);
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) o[t] *= inv;
+    }
+    if (pos < 0) return;
+#pragma unroll
+    for (int t = 0; t < DVB; ++t) {
+        if (t * 16 >= a.dv) continue;
+        const int e = t * 16 + quad * 4;
+        short4v packed;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = o[t][i];
+            if (a.gate) v = v / (1.f + expf(-a.gate[(size_t)tok * a.gate_stride + a.gate_column + (size_t)head * a.dv + e + i]));
+            packed[i] = bits_of((__bf16)v);
+        }
+        *reinterpret_cast<short4v*>(a.out + ((size_t)tok * a.heads + head) * a.dv + e) = packed;
+    }
+}
+
+template <int DSTEPS, int DVB, int MAPS>
+__global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(MaskedArgs a) {
+    __shared__ float meet[MB_WAVES - 1][kWave][DVB * 4 + 2];
+    const int* tile = a.tiles + 4 * blockIdx.x;
+    const int t0 = tile[0], n = tile[1], r = tile[2], p0 = tile[3];
+    const int g = blockIdx.y, group = a.heads / a.kv_heads;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), col = lane & 15;
+    const int* table = a.block_table + (size_t)r * a.max_blocks;
+    auto first_key = [&](int p) {
+        int lo = 0;
+        if (a.chunk > 0) lo = p - p % a.chunk;
+        if (a.window > 0) lo = max(lo, p - a.window + 1);
+        return lo;
+    };
+    const bool lone = n == 1;
+    // head places of a pass (a power of two up to the waves), and the waves that share a place's keys
+    int places = 1;
+    if (!lone)
+        while (places < group && places < MB_WAVES) places *= 2;
+    const int splits = MB_WAVES / places;
+    const int place = wave % places, split = wave / places;
+    // the blocks from the first token's first key to the last token
+    const int first = first_key(p0) / 16, last = (p0 + n - 1) / 16;
+    const int heads_a_pass = lone ? 16 : places;
+    ColumnState<DVB, MAPS> st;
+    for (int h0 = 0; h0 < group; h0 += heads_a_pass) {
+        // the lane's column: a token of the tile for the wave's head, or a head of the group for the lone token
+        const int hh = lone ? h0 + col : h0 + place;
+        const bool on = hh < group && (lone || col < n);
+        const int head = g * group + (hh < group ? hh : 0);
+        const int tok = lone ? t0 : t0 + (col < n ? col : 0);
+        const int pos = on ? (lone ? p0 : p0 + col) : -1;
+        const int lo = on ? first_key(pos) : 0;
+        const bool wave_on = lone || h0 + place < group;
+        if (wave_on)
+            attend_blocks<DSTEPS, DVB, MAPS>(st, a, g, tok, head, pos, lo, table, first + split, last, splits, lane);
+        if (splits > 1) {
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m) {
+                __syncthreads();            // the rows of the map before this one have been taken in
+                if (split > 0 && wave_on) {
+                    float* mine = meet[wave - places][lane];
+                    mine[0] = st.m[m];
+                    mine[1] = st.l[m];
+#pragma unroll
+                    for (int t = 0; t < DVB; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) mine[2 + t * 4 + i] = st.o[m][t][i];
+                }
+                __syncthreads();
+                if (split == 0 && wave_on)
+                    for (int w = 1; w < splits; ++w) {          // in the waves' order
+                        const float* its = meet[place + w * places - places][lane];
+                        const float m_new = fmaxf(st.m[m], its[0]);
+                        const float base = m_new == -INFINITY ? 0.f : m_new;
+                        const float mine_by = expf(st.m[m] - base), its_by = expf(its[0] - base);
+                        st.l[m] = fmaf(st.l[m], mine_by, its[1] * its_by);
+#pragma unroll
+                        for (int t = 0; t < DVB; ++t)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                st.o[m][t][i] = fmaf(st.o[m][t][i], mine_by, its[2 + t * 4 + i] * its_by);
+                        st.m[m] = m_new;
+                    }
+            }
+        }
+        if (split == 0 && wave_on) finish_column<DVB, MAPS>(st, a, tok, head, pos, lane);
+    }
+}
+
+}  // namespace lc
+
+using namespace lc;
+
+// Whether the matrix-core kernel takes these sizes (else the general kernel serves them).
+LC_API int lc_masked_attention_bf16_supported(int d, int dv, int page_size, int maps) {
+    return d > 0 && d % 8 == 0 && d <= 128 && dv > 0 && dv % 16 == 0 && dv <= 128 && page_size > 0 && page_size % 16 == 0
+           && (maps == 1 || maps == 2);
+}
+
+// tiles int32 [num_tiles, 4]: first token row, tokens (1..16), request, first position
+LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const void* v_cache, const int* tiles,
+                                    int num_tiles, const int* block_table, int max_blocks, int page_size, int heads,
+                                    int kv_heads, int maps, int d, int dv, float scale, int chunk, int window,
+                                    const float* r1, const float* r2, const float* sink, float lambda, int unit_out,
+                                    float eps, float out_scale, const float* gate, int gate_stride, int gate_column,
+                                    void* out, hipStream_t stream) {
+    LC_CHECK(num_tiles >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && max_blocks > 0,
+             "masked attention: bad sizes");
+    LC_CHECK(lc_masked_attention_bf16_supported(d, dv, page_size, maps),
+             "masked attention on the matrix cores: sizes d=%d dv=%d page=%d maps=%d are not taken", d, dv, page_size, maps);
+    if (num_tiles == 0) return 0;
+    LC_CHECK(q && k_cache && v_cache && tiles && block_table && out, "masked attention: null pointer");
+    LC_CHECK((r1 == nullptr) == (r2 == nullptr), "masked attention: the bias needs both of its vectors");
+    LC_CHECK(kv_heads <= 65535, "masked attention: too many kv heads");
+    MaskedArgs a{(const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, tiles, block_table, max_blocks, page_size,
+                 heads, kv_heads, d, dv, scale, chunk, window, r1, r2, sink, lambda, unit_out, eps, out_scale, gate,
+                 gate_stride, gate_column, (bf16*)out};
+    const dim3 grid(num_tiles, kv_heads);
+    const int dsteps = (d + 31) / 32, dvb = dv / 16;
+#define LC_MB(DS, VB)                                                                                  \
+    do {                                                                                               \
+        if (maps == 1) masked_attention_bf16_kernel<DS, VB, 1><<<grid, MB_THREADS, 0, stream>>>(a);    \
+        else masked_attention_bf16_kernel<DS, VB, 2><<<grid, MB_THREADS, 0, stream>>>(a);              \
+    } while (0)
+#define LC_MB_DV(DS)                     \
+    do {                                 \
+        if (dvb <= 2) LC_MB(DS, 2);      \
+        else if (dvb <= 4) LC_MB(DS, 4); \
+        else LC_MB(DS, 8);               \
+    } while (0)
+    if (dsteps <= 2) LC_MB_DV(2);
+    else LC_MB_DV(4);
+#undef LC_MB_DV
+#undef LC_MB
+    LC_LAUNCH_CHECK("masked_attention_bf16");
+    return 0;
+}

@@ -104,7 +104,9 @@ _SIGNATURES = {
     "lc_moe_combine_shared": "pppiiipipiipip",
     "lc_gated_activation_weighted": "ppippiiip",
     "lc_masked_attention": "pppi" + "ppp" + "ii" + "i" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
-    "lc_attention_prepare": "p" + "iiiiiii" + "pip" + "ppp" + "pip" + "if" + "ppp" + "i" + "pp",
+    "lc_attention_prepare": "p" + "iiiiiii" + "pip" + "ppp" + "pip" + "if" + "ppp" + "i" + "pip",
+    "lc_masked_attention_bf16_supported": "iiii",
+    "lc_masked_attention_bf16": "ppp" + "pi" + "pii" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
     "lc_state_space_prepare": "piiiiii" + "ppi" + "ppp" + "ppp" + "pp" + "p",
     "lc_state_space_readout": "pppiipiipifipip",
     "lc_scaled_sum": "pifpifpqp",
@@ -1791,6 +1793,28 @@ MASKED_ATTENTION_MAX = 256      # entries of a key head and of a value head at m
 SHORT_CONV_MAX_TAPS = 8
 
 
+class _MaskedSwitch(threading.local):
+    on = True
+
+
+_masked_fast = _MaskedSwitch()
+
+
+def masked_attention_matrix_cores(on: bool) -> bool:
+    """Tests and tuning: whether :func:`masked_attention` may take the matrix-core kernel (for the calling
+    thread).  Returns the setting before."""
+    before = _masked_fast.on
+    _masked_fast.on = bool(on)
+    return before
+
+
+def masked_attention_on_matrix_cores(dtype: torch.dtype, d: int, dv: int, page_size: int, maps: int) -> bool:
+    """Whether the matrix-core kernel serves these sizes: bfloat16, key heads of a multiple of 8 up to 128 entries,
+    value heads of a multiple of 16 up to 128, pages of a multiple of 16 tokens."""
+    return dtype == torch.bfloat16 and bool(library().lc_masked_attention_bf16_supported(int(d), int(dv), int(page_size),
+                                                                                        int(maps)))
+
+
 def attention_prepare(proj: torch.Tensor, nq: int, nk: int, nv: int, d: int, dv: int, out_dtype: torch.dtype,
                       k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                       rows: Optional[torch.Tensor], taps: Optional[torch.Tensor] = None,
@@ -1803,8 +1827,9 @@ def attention_prepare(proj: torch.Tensor, nq: int, nk: int, nv: int, d: int, dv:
     inputs from before the step come from ``tail`` float32 [slots, K - 1, columns] (the request's last K - 1
     inputs, oldest first).  ``table`` float32 [positions, rot] (cosines | sines): entries 2i, 2i + 1 of the first
     ``rot`` of every q and k head are rotated by angle i of the token's position.  ``unit_eps``: every q and k
-    head is divided by its root mean square.  Returns q [T, nq d] of ``out_dtype``; k and v go to row ``rows[t]``
-    of ``k_cache`` [rows, nk d] and ``v_cache`` [rows, nv dv] (where ``rows`` is given and not negative)."""
+    head is divided by its root mean square.  Returns q [T, nq d] of ``out_dtype``; k and v go to place ``rows[t]``
+    (page * page size + place in the page; where ``rows`` is given and not negative) of ``k_cache`` [pages, page,
+    nk d] and ``v_cache`` [pages, nv dv, page]."""
     _need(proj, "attention_prepare proj", torch.float32, 2)
     T, cols = proj.shape
     C = (nq + nk) * d + nv * dv
@@ -1833,14 +1858,16 @@ def attention_prepare(proj: torch.Tensor, nq: int, nk: int, nv: int, d: int, dv:
         _need(rows, "cache rows", torch.int32, 1)
         if k_cache is None or v_cache is None or k_cache.dtype != out_dtype or v_cache.dtype != out_dtype:
             raise KernelError("attention_prepare: the cache must have the queries' dtype")
-        if k_cache.shape[-1] != nk * d or v_cache.shape[-1] != nv * dv:
-            raise KernelError("attention_prepare: the cache rows do not fit the heads")
+        if k_cache.dim() != 3 or v_cache.dim() != 3 or k_cache.shape[2] != nk * d or v_cache.shape[1] != nv * dv \
+                or v_cache.shape[2] != k_cache.shape[1] or v_cache.shape[0] != k_cache.shape[0]:
+            raise KernelError("attention_prepare: the cache does not fit the heads")
     q = torch.empty((T, nq * d), dtype=out_dtype, device=proj.device)
     if T:
         _call("lc_attention_prepare", _ptr(proj), cols, T, nq, nk, nv, d, dv, _ptr(taps), K, _ptr(tail),
               _ptr(tok_req), _ptr(q_offsets), _ptr(slot_ids), _ptr(table), int(rot), _ptr(positions),
               0 if unit_eps is None else 1, float(unit_eps or 0.0), _ptr(q), _ptr(k_cache if rows is not None else None),
-              _ptr(v_cache if rows is not None else None), _dt(q), _ptr(rows), _stream())
+              _ptr(v_cache if rows is not None else None), _dt(q), _ptr(rows),
+              k_cache.shape[1] if rows is not None else 0, _stream())
     return q
 
 
@@ -1849,7 +1876,8 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      maps: int, d: int, dv: int, scale: float, chunk: int = 0, window: int = 0,
                      r1: Optional[torch.Tensor] = None, r2: Optional[torch.Tensor] = None,
                      sink: Optional[torch.Tensor] = None, subtract: float = 0.0, unit_eps: Optional[float] = None,
-                     out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, gate_column: int = 0) -> torch.Tensor:
+                     out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, gate_column: int = 0,
+                     plan=None) -> torch.Tensor:
     """Attention of every token of the batch over its request's cached keys lo .. p (p its position; lo the start
     of its chunk of ``chunk`` positions, of its window of ``window``, or 0), float32 arithmetic.  ``q`` [T, heads
     maps d]; ``k_cache`` [pages, page, kv_heads maps d], ``v_cache`` [pages, page, kv_heads dv].  Scores are
@@ -1857,16 +1885,18 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     exp(sink[h]) to the softmax's denominator.  ``maps`` = 2: a head's two maps over the same values are combined as
     a_0 - ``subtract`` a_1.  ``unit_eps``: the head's output is divided by its root mean square and multiplied by
     ``out_scale``.  ``gate`` float32 [T, >= gate_column + heads dv]: the output times sigmoid of those columns.
+    ``plan``: the step's tiles (:func:`plan_latent_attention`: up to 16 tokens of one request each); with them,
+    bfloat16 operands of sizes the matrix-core kernel takes (:func:`masked_attention_on_matrix_cores`) go there.
     -> [T, heads dv] in q's dtype."""
     _need(q, "masked_attention q", None, 2)
     T = q.shape[0]
     if q.shape[1] != heads * maps * d:
         raise KernelError(f"masked_attention: q has {q.shape[1]} columns, expected {heads * maps * d}")
-    for cache, width, what in ((k_cache, kv_heads * maps * d, "keys"), (v_cache, kv_heads * dv, "values")):
-        _need(cache, f"masked_attention {what}", q.dtype, 3)
-        if cache.shape[1] != page_size or cache.shape[2] != width:
-            raise KernelError(f"masked_attention: the {what} {tuple(cache.shape)} do not fit pages of {page_size} "
-                              f"rows of {width}")
+    _need(k_cache, "masked_attention keys", q.dtype, 3)
+    _need(v_cache, "masked_attention values", q.dtype, 3)
+    if tuple(k_cache.shape[1:]) != (page_size, kv_heads * maps * d) or tuple(v_cache.shape[1:]) != (kv_heads * dv, page_size):
+        raise KernelError(f"masked_attention: keys {tuple(k_cache.shape)} and values {tuple(v_cache.shape)} do not fit "
+                          f"pages of {page_size} with rows of {kv_heads * maps * d} and {kv_heads * dv}")
     _need(tok_req, "tok_req", torch.int32, 1)
     _need(positions, "positions", torch.int32, 1)
     _need(block_table, "block_table", torch.int32, 2)
@@ -1880,7 +1910,14 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         if gate.shape[0] != T or gate_column < 0 or gate_column + heads * dv > gate.shape[1]:
             raise KernelError("masked_attention: the gate does not fit the rows")
     out = torch.empty((T, heads * dv), dtype=q.dtype, device=q.device)
-    if T:
+    if T and plan is not None and _masked_fast.on and masked_attention_on_matrix_cores(q.dtype, d, dv, page_size, maps):
+        tiles = plan.arrays["tiles"]
+        _call("lc_masked_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tiles), tiles.shape[0],
+              _ptr(block_table), block_table.shape[1], int(page_size), heads, kv_heads, maps, d, dv, float(scale),
+              int(chunk), int(window), _ptr(r1), _ptr(r2), _ptr(sink), float(subtract), 0 if unit_eps is None else 1,
+              float(unit_eps or 0.0), float(out_scale), _ptr(gate), gate.shape[1] if gate is not None else 0,
+              int(gate_column), _ptr(out), _stream())
+    elif T:
         _call("lc_masked_attention", _ptr(q), _ptr(k_cache), _ptr(v_cache), _dt(q), _ptr(tok_req), _ptr(positions),
               _ptr(block_table), block_table.shape[1], int(page_size), T, heads, kv_heads, maps, d, dv, float(scale),
               int(chunk), int(window), _ptr(r1), _ptr(r2), _ptr(sink), float(subtract), 0 if unit_eps is None else 1,

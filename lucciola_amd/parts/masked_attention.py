@@ -17,7 +17,9 @@
   start; ``window``: only the last so many positions.
 
 The projections leave as float32; one kernel makes q, k and v of them (convolution, rotation, unit norm) and
-writes k and v into the cache's rows; the attention kernel computes in float32 whatever the cache's type.
+writes k and v into the cache (keys token-major, values transposed inside a page).  Scores, softmax, bias, sink
+and the maps' combination are float32 whatever the cache's type; with a bfloat16 cache of sizes that fit, the two
+products run on the matrix cores (``ops.masked_attention``), else in float32 multiply-adds.
 """
 from __future__ import annotations
 
@@ -122,6 +124,10 @@ class MaskedAttention(Part):
             return rows, FixedStates(((self.taps - 1, self.channels),))
         return rows
 
+    def batch_planner(self):
+        # the step's tokens in tiles of up to 16 of one request: the matrix-core kernel's work items
+        return ops.LATENT_PLAN, ops.plan_latent_attention
+
     def tables_epoch(self) -> int:
         return self.position.tables_epoch() if self.position is not None else 0
 
@@ -140,7 +146,7 @@ class MaskedAttention(Part):
             table, rot = self.position.rotary_table(batch.max_position), self.position.rotary_dim
         q = ops.attention_prepare(
             proj, self.nh * self.maps, self.nkv * self.maps, self.nkv, self.d, self.dv, self.dtype,
-            k_cache.view(-1, self.nk_cols), v_cache.view(-1, self.nv_cols), pages.slots if site.writes_cache else None,
+            k_cache, v_cache, pages.slots if site.writes_cache else None,
             taps=self.conv, tail=tail, tok_req=batch.tok_req, q_offsets=batch.q_offsets, slot_ids=batch.slot_ids,
             table=table, rot=rot, positions=batch.positions, unit_eps=self.eps if self.unit_qk else None)
         if self.taps > 1:
@@ -151,5 +157,5 @@ class MaskedAttention(Part):
             self.maps, self.d, self.dv, self.scale, chunk=self.chunk, window=self.window, r1=self.r1, r2=self.r2,
             sink=self.sink, subtract=self.subtract, unit_eps=self.eps if self.maps == 2 else None,
             out_scale=1.0 - self.difference if self.maps == 2 else 1.0,
-            gate=proj if self.has_gate else None, gate_column=self.channels)
+            gate=proj if self.has_gate else None, gate_column=self.channels, plan=batch.plans.get(ops.LATENT_PLAN))
         return ops.gemm(o, self.o, self.dtype, defer=True)

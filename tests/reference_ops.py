@@ -582,18 +582,20 @@ def attention_prepare(proj, nq, nk, nv, d, dv, out_dtype, k_cache, v_cache, rows
     if unit_eps is not None:
         qk = qk / torch.sqrt((qk * qk).mean(-1, keepdim=True) + unit_eps)
     if rows is not None:
+        page = k_cache.shape[1]
         keep = rows >= 0
-        k_cache[rows[keep].long()] = qk[keep, nq:].reshape(-1, nk * d).to(k_cache.dtype)
-        v_cache[rows[keep].long()] = y[keep, (nq + nk) * d:].to(v_cache.dtype)
+        at = rows[keep].long()
+        k_cache[at // page, at % page] = qk[keep, nq:].reshape(-1, nk * d).to(k_cache.dtype)
+        v_cache[at // page, :, at % page] = y[keep, (nq + nk) * d:C].to(v_cache.dtype)      # transposed inside a page
     return qk[:, :nq].reshape(T, nq * d).to(out_dtype)
 
 
 def masked_attention(q, k_cache, v_cache, tok_req, positions, block_table, page_size, heads, kv_heads, maps, d, dv,
                      scale, chunk=0, window=0, r1=None, r2=None, sink=None, subtract=0.0, unit_eps=None,
-                     out_scale=1.0, gate=None, gate_column=0):
+                     out_scale=1.0, gate=None, gate_column=0, plan=None):
     T = q.shape[0]
     kc = k_cache.reshape(-1, kv_heads, maps, d).to(F64)
-    vc = v_cache.reshape(-1, kv_heads, dv).to(F64)
+    vc = v_cache.transpose(1, 2).reshape(-1, kv_heads, dv).to(F64)
     qq = q.to(F64).view(T, heads, maps, d)
     out = torch.zeros(T, heads, dv, dtype=F64)
     for t in range(T):

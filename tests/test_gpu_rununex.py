@@ -124,6 +124,15 @@ def request_lists(lengths, slots):
     return tok_req, q_offsets, torch.tensor(slots, dtype=torch.int32)
 
 
+def tiles_of(step):
+    """The step's tokens in tiles of up to 16 of one request, as the engine's planner makes them, on the GPU."""
+    from lucciola_amd.engine.batch import HostLayout, Plan
+    layout = HostLayout(len(step.new), sum(step.new), step.q_offsets.tolist(), list(step.cached), step.page,
+                        all(n == 1 for n in step.new))
+    arrays, info = ops.plan_latent_attention(layout)
+    return Plan({k: torch.from_numpy(v).to(DEV) for k, v in arrays.items()}, info)
+
+
 class PagedStep:
     """Requests with some tokens cached already and some new ones, pages handed out in a shuffled order."""
 
@@ -159,6 +168,12 @@ ATTENTION_CASES = [
     (6, 2, 1, 7, 9, 8, 5, 0, 0, 0, True, True, True, True),
     (2, 2, 1, 32, 16, 16, 0, 33, 4, 0, False, True, False, False),
     (2, 1, 2, 128, 256, 32, 300, 0, 1, 64, False, False, True, False),
+    # sizes that the matrix-core kernel takes
+    (8, 2, 2, 64, 128, 16, 100, 0, 4, 64, False, False, False, False),
+    (4, 4, 2, 48, 96, 16, 0, 0, 2, 48, False, False, False, False),
+    (16, 4, 1, 128, 128, 16, 64, 0, 0, 0, True, True, True, True),
+    (20, 1, 1, 64, 64, 32, 0, 90, 0, 0, True, True, True, True),
+    (2, 2, 1, 24, 16, 48, 33, 0, 0, 8, False, False, True, False),
 ]
 
 
@@ -176,10 +191,10 @@ def test_prepare_and_masked_attention(case_, dtype):
     cols = C + (heads * dv if gate else 0)
     proj = torch.randn(T, cols, generator=g)
     k_cache = torch.zeros(step.pages, page, nk * d, dtype=dtype)
-    v_cache = torch.zeros(step.pages, page, nv * dv, dtype=dtype)
-    old = step.old_rows()
+    v_cache = torch.zeros(step.pages, nv * dv, page, dtype=dtype)
+    old = torch.tensor(step.old_rows())
     k_cache.view(-1, nk * d)[old] = torch.randn(len(old), nk * d, generator=g).to(dtype)
-    v_cache.view(-1, nv * dv)[old] = torch.randn(len(old), nv * dv, generator=g).to(dtype)
+    v_cache[old // page, :, old % page] = torch.randn(len(old), nv * dv, generator=g).to(dtype)
     conv = torch.randn(C, taps, generator=g) * 0.6 if taps else None
     tail = torch.randn(5, max(taps - 1, 0), C, generator=g) if taps > 1 else None
     table = None
@@ -196,7 +211,7 @@ def test_prepare_and_masked_attention(case_, dtype):
         kc, vc, tl = on(k_cache), on(v_cache), on(tail)
         lists = dict(tok_req=on(step.tok_req), q_offsets=on(step.q_offsets), slot_ids=on(step.slot_ids))
         pj = on(proj)
-        q = o.attention_prepare(pj, nq, nk, nv, d, dv, dtype, kc.view(-1, nk * d), vc.view(-1, nv * dv), on(step.rows),
+        q = o.attention_prepare(pj, nq, nk, nv, d, dv, dtype, kc, vc, on(step.rows),
                                 taps=on(conv), tail=tl, table=on(table), rot=rot, positions=on(step.positions),
                                 unit_eps=1e-5 if unit else None, **lists)
         if taps > 1:
@@ -205,10 +220,19 @@ def test_prepare_and_masked_attention(case_, dtype):
                                  d, dv, 0.21, chunk=chunk, window=window, r1=on(r1), r2=on(r2), sink=on(sinks),
                                  subtract=0.45, unit_eps=1e-5 if maps == 2 else None, out_scale=0.7,
                                  gate=pj if gate else None, gate_column=C)
-        outs.append([t.cpu() if t is not None else None for t in (q, kc, vc, tl, out)])
-    for got, want, what in zip(outs[1], outs[0], ("q", "key rows", "value rows", "tails", "attention")):
-        if want is not None:
-            close(got, want, torch.float32 if what == "tails" else dtype, what, 3.0 if what == "attention" else 1.0)
+        fast = None
+        if o is ops and ops.masked_attention_on_matrix_cores(dtype, d, dv, page, maps):
+            fast = o.masked_attention(q, kc, vc, lists["tok_req"], on(step.positions), on(step.table), page, heads, kv,
+                                      maps, d, dv, 0.21, chunk=chunk, window=window, r1=on(r1), r2=on(r2), sink=on(sinks),
+                                      subtract=0.45, unit_eps=1e-5 if maps == 2 else None, out_scale=0.7,
+                                      gate=pj if gate else None, gate_column=C, plan=tiles_of(step))
+        outs.append([t.cpu() if t is not None else None for t in (q, kc, vc, tl, out, fast)])
+    if dtype == torch.bfloat16 and case_ in ATTENTION_CASES[6:]:
+        assert outs[1][5] is not None, "the matrix-core kernel should take these sizes"
+    for got, want, what in zip(outs[1], outs[0] + [outs[0][4]], ("q", "key rows", "value rows", "tails", "attention",
+                                                                  "attention on the matrix cores")):
+        if want is not None and got is not None:
+            close(got, want, torch.float32 if what == "tails" else dtype, what, 3.0 if "attention" in what else 1.0)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -217,28 +241,37 @@ def test_one_key_carries_the_weight(dtype, chunk, window, page):
     """Among hundreds of keys one has a score that stands out; its value is one-hot.  A query sees it exactly when it
     lies inside the query's chunk or window: the key at the edge just inside, the one just outside, far keys, and the
     first tokens of a sequence; prompts and lone tokens alike."""
-    heads, d, dv = 2, 16, 8
+    heads, d, dv = 2, 16, 16
     length = 330
     k_rows = torch.zeros(length, heads * d)
     v_rows = torch.zeros(length, heads * dv)
     v_rows[:, :] = -1.0
     step = PagedStep([0], [length], page, seed=chunk + window)
     k_cache = torch.zeros(step.pages, page, heads * d, dtype=dtype, device=DEV)
-    v_cache = torch.zeros(step.pages, page, heads * dv, dtype=dtype, device=DEV)
+    v_cache = torch.zeros(step.pages, heads * dv, page, dtype=dtype, device=DEV)
+    places = step.rows.long().to(DEV)
     for marked in (0, 1, 39, 40, 41, 279, 280, 299, 300, 305, 329):
         k = k_rows.clone()
         k[marked, :] = 1.0
         v = v_rows.clone()
         v[marked] = 5.0
-        k_cache.view(-1, heads * d)[step.rows.long()] = k.to(dtype).to(DEV)
-        v_cache.view(-1, heads * dv)[step.rows.long()] = v.to(dtype).to(DEV)
+        k_cache.view(-1, heads * d)[places] = k.to(dtype).to(DEV)
+        v_cache[places // page, :, places % page] = v.to(dtype).to(DEV)
         q = torch.ones(length, heads * d, dtype=dtype, device=DEV)
-        for lone in (False, True):
+        for lone, fast in ((False, False), (True, False), (False, True), (True, True)):
             rows = list(range(length)) if not lone else [marked, min(marked + 1, length - 1), length - 1]
             pos = torch.tensor(rows, dtype=torch.int32, device=DEV)
+            plan = None
+            if fast:        # the same on the matrix cores: the prompt in tiles of 16, or lone tokens of three requests
+                if not ops.masked_attention_on_matrix_cores(dtype, d, dv, page, 1):
+                    continue
+                from lucciola_amd.engine.batch import Plan
+                tiles = [[t0, min(16, length - t0), 0, t0] for t0 in range(0, length, 16)] if not lone else \
+                    [[i, 1, 0, p] for i, p in enumerate(rows)]
+                plan = Plan({"tiles": torch.tensor(tiles, dtype=torch.int32, device=DEV)}, {})
             out = ops.masked_attention(q[:len(rows)].contiguous(), k_cache, v_cache,
                                        torch.zeros(len(rows), dtype=torch.int32, device=DEV), pos, step.table.to(DEV), page,
-                                       heads, heads, 1, d, dv, 4.0, chunk=chunk, window=window).float().cpu()
+                                       heads, heads, 1, d, dv, 4.0, chunk=chunk, window=window, plan=plan).float().cpu()
             for at, p in enumerate(rows):
                 lo = 0
                 if chunk:
@@ -247,7 +280,8 @@ def test_one_key_carries_the_weight(dtype, chunk, window, page):
                     lo = max(lo, p - window + 1)
                 sees = lo <= marked <= p
                 want = 5.0 if sees else -1.0
-                assert abs(float(out[at, 0]) - want) < 1e-2, (f"key {marked}, query {p} ({'lone' if lone else 'prompt'}): "
+                assert abs(float(out[at, 0]) - want) < 1e-2, (f"key {marked}, query {p} ({'lone' if lone else 'prompt'}, "
+                                                              f"{'matrix cores' if fast else 'general'}): "
                                                               f"{float(out[at, 0]):.3f}, expected {want}")
 
 
