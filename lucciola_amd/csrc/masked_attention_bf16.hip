@@ -12,6 +12,9 @@
 //   A lone token: the 16 columns are query heads of the group, and all eight waves share out the blocks.
 // Waves that shared a column's keys leave their maxima, sums and rows in LDS, and the first of them takes the
 // others in, in their order.  A wave asks for the next block's keys before it works on this one's.
+// In a step of lone tokens only, with fewer workgroups than the card has room for, a token's blocks are also
+// shared out over several workgroups (the grid's last place); each leaves its joined sums in a workspace, and a
+// second kernel takes them in, in their order, and finishes the columns.
 // Keys are walked in blocks of 16 (one part of a page).  S^T = K Q^T (16x16x32: a lane's operand is 16 bytes
 // in a row of a key, straight from memory) leaves a lane with four keys of one query column, which is the
 // operand P^T of O^T += V^T P^T (16x16x16; V^T's operand is four neighbouring keys of one value entry, 8
@@ -45,7 +48,12 @@ struct MaskedArgs {
     const float* gate;
     int gate_stride, gate_column;
     bf16* out;
+    float* shares;      // where a lone token's keys are shared out over workgroups: their sums, joined by a second kernel
+    int zsplits;
 };
+
+// floats a wave leaves per lane and map where key ranges are joined: maximum, sum, the lane's part of O^T
+template <int DVB> constexpr int share_floats() { return DVB * 4 + 2; }
 
 __device__ __forceinline__ short bits_of(__bf16 v) { return __builtin_bit_cast(short, v); }
 
@@ -245,6 +253,8 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
         return lo;
     };
     const bool lone = n == 1;
+    const int z = blockIdx.z, zsplits = lone ? a.zsplits : 1;
+    if (!lone && z > 0) return;
     // head places of a pass (a power of two up to the waves), and the waves that share a place's keys
     int places = 1;
     if (!lone)
@@ -265,7 +275,8 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
         const int lo = on ? first_key(pos) : 0;
         const bool wave_on = lone || h0 + place < group;
         if (wave_on)
-            attend_blocks<DSTEPS, DVB, MAPS>(st, a, g, tok, head, pos, lo, table, first + split, last, splits, lane);
+            attend_blocks<DSTEPS, DVB, MAPS>(st, a, g, tok, head, pos, lo, table, first + z * splits + split, last,
+                                             splits * zsplits, lane);
         if (splits > 1) {
 #pragma unroll
             for (int m = 0; m < MAPS; ++m) {
@@ -296,7 +307,64 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
                     }
             }
         }
-        if (split == 0 && wave_on) finish_column<DVB, MAPS>(st, a, tok, head, pos, lane);
+        if (split == 0 && wave_on) {
+            if (zsplits > 1) {
+                const int passes = (group + 15) / 16;
+                float* mine = a.shares + ((((size_t)blockIdx.x * a.kv_heads + g) * passes + h0 / 16) * zsplits + z)
+                                             * kWave * MAPS * share_floats<DVB>() + (size_t)lane * MAPS * share_floats<DVB>();
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m) {
+                    mine[m * share_floats<DVB>()] = st.m[m];
+                    mine[m * share_floats<DVB>() + 1] = st.l[m];
+#pragma unroll
+                    for (int t = 0; t < DVB; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) mine[m * share_floats<DVB>() + 2 + t * 4 + i] = st.o[m][t][i];
+                }
+            } else {
+                finish_column<DVB, MAPS>(st, a, tok, head, pos, lane);
+            }
+        }
+    }
+}
+
+// One wave per lone token and kv head: the workgroups' shares taken in, in their order; then the columns' end.
+template <int DVB, int MAPS>
+__global__ __launch_bounds__(kWave) void masked_attention_bf16_join_kernel(MaskedArgs a) {
+    const int* tile = a.tiles + 4 * blockIdx.x;
+    const int t0 = tile[0], n = tile[1], p0 = tile[3];
+    if (n != 1) return;
+    const int g = blockIdx.y, group = a.heads / a.kv_heads, lane = threadIdx.x, col = lane & 15;
+    const int passes = (group + 15) / 16;
+    for (int h0 = 0; h0 < group; h0 += 16) {
+        const bool on = h0 + col < group;
+        const int head = g * group + (on ? h0 + col : 0);
+        ColumnState<DVB, MAPS> st;
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) {
+            st.m[m] = -INFINITY;
+            st.l[m] = 0.f;
+#pragma unroll
+            for (int t = 0; t < DVB; ++t) st.o[m][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+        for (int z = 0; z < a.zsplits; ++z) {
+            const float* its = a.shares + ((((size_t)blockIdx.x * a.kv_heads + g) * passes + h0 / 16) * a.zsplits + z)
+                                              * kWave * MAPS * share_floats<DVB>() + (size_t)lane * MAPS * share_floats<DVB>();
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m) {
+                const float* row = its + m * share_floats<DVB>();
+                const float m_new = fmaxf(st.m[m], row[0]);
+                const float base = m_new == -INFINITY ? 0.f : m_new;
+                const float mine_by = expf(st.m[m] - base), its_by = expf(row[0] - base);
+                st.l[m] = fmaf(st.l[m], mine_by, row[1] * its_by);
+#pragma unroll
+                for (int t = 0; t < DVB; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) st.o[m][t][i] = fmaf(st.o[m][t][i], mine_by, row[2 + t * 4 + i] * its_by);
+                st.m[m] = m_new;
+            }
+        }
+        finish_column<DVB, MAPS>(st, a, t0, head, on ? p0 : -1, lane);
     }
 }
 
@@ -310,13 +378,23 @@ LC_API int lc_masked_attention_bf16_supported(int d, int dv, int page_size, int 
            && (maps == 1 || maps == 2);
 }
 
-// tiles int32 [num_tiles, 4]: first token row, tokens (1..16), request, first position
+// float32 words of workspace for a step of `num_tiles` lone tokens whose keys are shared out over `zsplits` workgroups
+LC_API long long lc_masked_attention_bf16_workspace(int num_tiles, int heads, int kv_heads, int maps, int dv, int zsplits) {
+    if (num_tiles <= 0 || kv_heads <= 0 || heads % kv_heads || zsplits <= 1) return 0;
+    const int dvb = dv <= 32 ? 2 : (dv <= 64 ? 4 : 8), passes = (heads / kv_heads + 15) / 16;
+    return (long long)num_tiles * kv_heads * passes * zsplits * kWave * maps * (dvb * 4 + 2);
+}
+
+// tiles int32 [num_tiles, 4]: first token row, tokens (1..16), request, first position.  zsplits > 1 (a step of lone
+// tokens only): every token's key blocks are shared out over that many workgroups, through `shares`
+// (lc_masked_attention_bf16_workspace words)
 LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const void* v_cache, const int* tiles,
                                     int num_tiles, const int* block_table, int max_blocks, int page_size, int heads,
                                     int kv_heads, int maps, int d, int dv, float scale, int chunk, int window,
                                     const float* r1, const float* r2, const float* sink, float lambda, int unit_out,
                                     float eps, float out_scale, const float* gate, int gate_stride, int gate_column,
-                                    void* out, hipStream_t stream) {
+                                    void* out, float* shares, int zsplits, hipStream_t stream) {
+    LC_CHECK(zsplits >= 1 && zsplits <= 64 && (zsplits == 1 || shares), "masked attention: bad shares");
     LC_CHECK(num_tiles >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && max_blocks > 0,
              "masked attention: bad sizes");
     LC_CHECK(lc_masked_attention_bf16_supported(d, dv, page_size, maps),
@@ -327,13 +405,18 @@ LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const vo
     LC_CHECK(kv_heads <= 65535, "masked attention: too many kv heads");
     MaskedArgs a{(const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, tiles, block_table, max_blocks, page_size,
                  heads, kv_heads, d, dv, scale, chunk, window, r1, r2, sink, lambda, unit_out, eps, out_scale, gate,
-                 gate_stride, gate_column, (bf16*)out};
-    const dim3 grid(num_tiles, kv_heads);
+                 gate_stride, gate_column, (bf16*)out, shares, zsplits};
+    const dim3 grid(num_tiles, kv_heads, zsplits), join_grid(num_tiles, kv_heads);
     const int dsteps = (d + 31) / 32, dvb = dv / 16;
-#define LC_MB(DS, VB)                                                                                  \
-    do {                                                                                               \
-        if (maps == 1) masked_attention_bf16_kernel<DS, VB, 1><<<grid, MB_THREADS, 0, stream>>>(a);    \
-        else masked_attention_bf16_kernel<DS, VB, 2><<<grid, MB_THREADS, 0, stream>>>(a);              \
+#define LC_MB(DS, VB)                                                                                                   \
+    do {                                                                                                                \
+        if (maps == 1) {                                                                                                \
+            masked_attention_bf16_kernel<DS, VB, 1><<<grid, MB_THREADS, 0, stream>>>(a);                                \
+            if (zsplits > 1) masked_attention_bf16_join_kernel<VB, 1><<<join_grid, kWave, 0, stream>>>(a);              \
+        } else {                                                                                                        \
+            masked_attention_bf16_kernel<DS, VB, 2><<<grid, MB_THREADS, 0, stream>>>(a);                                \
+            if (zsplits > 1) masked_attention_bf16_join_kernel<VB, 2><<<join_grid, kWave, 0, stream>>>(a);              \
+        }                                                                                                               \
     } while (0)
 #define LC_MB_DV(DS)                     \
     do {                                 \

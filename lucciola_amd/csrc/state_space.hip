@@ -15,35 +15,38 @@ namespace lc {
 __device__ __forceinline__ float ss_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float ss_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-// One workgroup per token.  proj [T, cols]: x (heads dv) | B (groups N) | C (groups N) | z (heads dv) | dt (heads);
-// the first C = heads dv + 2 groups N columns pass the convolution.  coef [3, T, heads N]; x_out [T, heads dv]
+// A thread per output entry.  proj [T, cols]: x (heads dv) | B (groups N) | C (groups N) | z (heads dv) | dt (heads);
+// the first C = heads dv + 2 groups N columns pass the convolution.  Entry (t, i): i < heads dv is a channel of x;
+// the others are (head, n) pairs, whose thread makes the head's step and decay and its group's B and C at n (the
+// heads of a group each make their own copy of those two: a few multiply-adds against a trip through memory).
+// coef [3, T, heads N]; x_out [T, heads dv]
 __global__ void state_space_prepare_kernel(const float* __restrict__ proj, int cols, int T, int heads, int groups,
                                            int N, int dv, const float* __restrict__ taps, const float* __restrict__ bias,
                                            int K, const float* __restrict__ tails, const float* __restrict__ dt_bias,
                                            const float* __restrict__ a_log, const int* __restrict__ tok_req,
                                            const int* __restrict__ q_offsets, const int* __restrict__ slot_ids,
                                            float* __restrict__ coef, float* __restrict__ x_out) {
-    extern __shared__ float bc[];            // B, then C, behind convolution and SiLU
-    const int t = blockIdx.x;
-    const int inner = heads * dv, C = inner + 2 * groups * N;
-    const int r = tok_req[t];
-    const int local = t - q_offsets[r];
-    const float* tail = K > 1 ? tails + (size_t)slot_ids[r] * (K - 1) * C : nullptr;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-        const float y = ss_silu(short_conv(proj, cols, t, local, c, taps, K, tail, C) + bias[c]);
-        if (c < inner) x_out[(size_t)t * inner + c] = y;
-        else bc[c - inner] = y;
-    }
-    __syncthreads();
-    const size_t plane = (size_t)T * heads * N;
-    const float* row = proj + (size_t)t * cols;
-    for (int i = threadIdx.x; i < heads * N; i += blockDim.x) {
-        const int head = i / N, n = i % N, g = head / (heads / groups);
-        const float step = ss_softplus(row[C + inner + head] + dt_bias[head]);
-        const size_t at = (size_t)t * heads * N + i;
+    const int inner = heads * dv, C = inner + 2 * groups * N, per_token = inner + heads * N;
+    const size_t total = (size_t)T * per_token, plane = (size_t)T * heads * N;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const int t = (int)(idx / per_token), i = (int)(idx % per_token);
+        const int r = tok_req[t];
+        const int local = t - q_offsets[r];
+        const float* tail = K > 1 ? tails + (size_t)slot_ids[r] * (K - 1) * C : nullptr;
+        if (i < inner) {
+            x_out[(size_t)t * inner + i] = ss_silu(short_conv(proj, cols, t, local, i, taps, K, tail, C) + bias[i]);
+            continue;
+        }
+        const int head = (i - inner) / N, n = (i - inner) % N, g = head / (heads / groups);
+        const int cb = inner + g * N + n, cc = inner + groups * N + g * N + n;
+        const float b = ss_silu(short_conv(proj, cols, t, local, cb, taps, K, tail, C) + bias[cb]);
+        const float c = ss_silu(short_conv(proj, cols, t, local, cc, taps, K, tail, C) + bias[cc]);
+        const float step = ss_softplus(proj[(size_t)t * cols + C + inner + head] + dt_bias[head]);
+        const size_t at = (size_t)t * heads * N + (i - inner);
         coef[at] = expf(-expf(a_log[head]) * step);
-        coef[plane + at] = step * bc[g * N + n];
-        coef[2 * plane + at] = bc[groups * N + g * N + n];
+        coef[plane + at] = step * b;
+        coef[2 * plane + at] = c;
     }
 }
 
@@ -96,10 +99,10 @@ LC_API int lc_state_space_prepare(const float* proj, int cols, int T, int heads,
     if (T == 0) return 0;
     LC_CHECK(proj && taps && bias && dt_bias && a_log && tok_req && q_offsets && slot_ids && coef && x_out && (K == 1 || tails),
              "state space prepare: null pointer");
-    const size_t lds = (size_t)2 * groups * N * sizeof(float);
-    LC_CHECK(lds <= 48 * 1024, "state space prepare: %d groups of %d state entries are too many", groups, N);
-    state_space_prepare_kernel<<<T, 256, lds, stream>>>(proj, cols, T, heads, groups, N, dv, taps, bias, K, tails, dt_bias,
-                                                        a_log, tok_req, q_offsets, slot_ids, coef, x_out);
+    const size_t total = (size_t)T * heads * (dv + N);
+    const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+    state_space_prepare_kernel<<<blocks, 256, 0, stream>>>(proj, cols, T, heads, groups, N, dv, taps, bias, K, tails, dt_bias,
+                                                           a_log, tok_req, q_offsets, slot_ids, coef, x_out);
     LC_LAUNCH_CHECK("state_space_prepare");
     return 0;
 }

@@ -106,7 +106,8 @@ _SIGNATURES = {
     "lc_masked_attention": "pppi" + "ppp" + "ii" + "i" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
     "lc_attention_prepare": "p" + "iiiiiii" + "pip" + "ppp" + "pip" + "if" + "ppp" + "i" + "pip",
     "lc_masked_attention_bf16_supported": "iiii",
-    "lc_masked_attention_bf16": "ppp" + "pi" + "pii" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
+    "lc_masked_attention_bf16": "ppp" + "pi" + "pii" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "ppip",
+    "lc_masked_attention_bf16_workspace": "iiiiii",
     "lc_state_space_prepare": "piiiiii" + "ppi" + "ppp" + "ppp" + "pp" + "p",
     "lc_state_space_readout": "pppiipiipifipip",
     "lc_scaled_sum": "pifpifpqp",
@@ -1800,6 +1801,21 @@ class _MaskedSwitch(threading.local):
 _masked_fast = _MaskedSwitch()
 
 
+class _MaskedSplits(threading.local):
+    forced = 0
+
+
+_masked_splits = _MaskedSplits()
+
+
+def masked_attention_force_splits(count: int) -> int:
+    """Tests and tuning: over how many workgroups a lone token's keys are shared out at most where a step allows
+    it (0: by the step's size; for the calling thread).  Returns the setting before."""
+    before = _masked_splits.forced
+    _masked_splits.forced = int(count)
+    return before
+
+
 def masked_attention_matrix_cores(on: bool) -> bool:
     """Tests and tuning: whether :func:`masked_attention` may take the matrix-core kernel (for the calling
     thread).  Returns the setting before."""
@@ -1877,7 +1893,7 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      r1: Optional[torch.Tensor] = None, r2: Optional[torch.Tensor] = None,
                      sink: Optional[torch.Tensor] = None, subtract: float = 0.0, unit_eps: Optional[float] = None,
                      out_scale: float = 1.0, gate: Optional[torch.Tensor] = None, gate_column: int = 0,
-                     plan=None) -> torch.Tensor:
+                     plan=None, max_ctx: int = 0) -> torch.Tensor:
     """Attention of every token of the batch over its request's cached keys lo .. p (p its position; lo the start
     of its chunk of ``chunk`` positions, of its window of ``window``, or 0), float32 arithmetic.  ``q`` [T, heads
     maps d]; ``k_cache`` [pages, page, kv_heads maps d], ``v_cache`` [pages, page, kv_heads dv].  Scores are
@@ -1886,8 +1902,9 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     a_0 - ``subtract`` a_1.  ``unit_eps``: the head's output is divided by its root mean square and multiplied by
     ``out_scale``.  ``gate`` float32 [T, >= gate_column + heads dv]: the output times sigmoid of those columns.
     ``plan``: the step's tiles (:func:`plan_latent_attention`: up to 16 tokens of one request each); with them,
-    bfloat16 operands of sizes the matrix-core kernel takes (:func:`masked_attention_on_matrix_cores`) go there.
-    -> [T, heads dv] in q's dtype."""
+    bfloat16 operands of sizes the matrix-core kernel takes (:func:`masked_attention_on_matrix_cores`) go there;
+    ``max_ctx`` (the longest request of the step) lets a step of few lone tokens share every token's keys out over
+    several workgroups.  -> [T, heads dv] in q's dtype."""
     _need(q, "masked_attention q", None, 2)
     T = q.shape[0]
     if q.shape[1] != heads * maps * d:
@@ -1912,11 +1929,20 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     out = torch.empty((T, heads * dv), dtype=q.dtype, device=q.device)
     if T and plan is not None and _masked_fast.on and masked_attention_on_matrix_cores(q.dtype, d, dv, page_size, maps):
         tiles = plan.arrays["tiles"]
+        # a step of lone tokens that leaves most of the card idle: every token's key blocks over several workgroups,
+        # a workgroup keeping two blocks a wave at least
+        zsplits, shares = 1, None
+        if not plan.info.get("any_portion", True) and max_ctx > 0:
+            reach = min(int(chunk) or max_ctx, int(window) or max_ctx, max_ctx)
+            zsplits = max(1, min(_masked_splits.forced or 512 // max(1, tiles.shape[0] * kv_heads), 16, reach // 256))
+            if zsplits > 1:
+                words = library().lc_masked_attention_bf16_workspace(tiles.shape[0], heads, kv_heads, maps, dv, zsplits)
+                shares = torch.empty((words,), dtype=torch.float32, device=q.device)
         _call("lc_masked_attention_bf16", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tiles), tiles.shape[0],
               _ptr(block_table), block_table.shape[1], int(page_size), heads, kv_heads, maps, d, dv, float(scale),
               int(chunk), int(window), _ptr(r1), _ptr(r2), _ptr(sink), float(subtract), 0 if unit_eps is None else 1,
               float(unit_eps or 0.0), float(out_scale), _ptr(gate), gate.shape[1] if gate is not None else 0,
-              int(gate_column), _ptr(out), _stream())
+              int(gate_column), _ptr(out), _ptr(shares), zsplits, _stream())
     elif T:
         _call("lc_masked_attention", _ptr(q), _ptr(k_cache), _ptr(v_cache), _dt(q), _ptr(tok_req), _ptr(positions),
               _ptr(block_table), block_table.shape[1], int(page_size), T, heads, kv_heads, maps, d, dv, float(scale),

@@ -157,5 +157,6 @@ class MaskedAttention(Part):
             self.maps, self.d, self.dv, self.scale, chunk=self.chunk, window=self.window, r1=self.r1, r2=self.r2,
             sink=self.sink, subtract=self.subtract, unit_eps=self.eps if self.maps == 2 else None,
             out_scale=1.0 - self.difference if self.maps == 2 else 1.0,
-            gate=proj if self.has_gate else None, gate_column=self.channels, plan=batch.plans.get(ops.LATENT_PLAN))
+            gate=proj if self.has_gate else None, gate_column=self.channels, plan=batch.plans.get(ops.LATENT_PLAN),
+            max_ctx=batch.max_ctx)
         return ops.gemm(o, self.o, self.dtype, defer=True)

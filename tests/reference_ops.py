@@ -592,7 +592,7 @@ def attention_prepare(proj, nq, nk, nv, d, dv, out_dtype, k_cache, v_cache, rows
 
 def masked_attention(q, k_cache, v_cache, tok_req, positions, block_table, page_size, heads, kv_heads, maps, d, dv,
                      scale, chunk=0, window=0, r1=None, r2=None, sink=None, subtract=0.0, unit_eps=None,
-                     out_scale=1.0, gate=None, gate_column=0, plan=None):
+                     out_scale=1.0, gate=None, gate_column=0, plan=None, max_ctx=0):
     T = q.shape[0]
     kc = k_cache.reshape(-1, kv_heads, maps, d).to(F64)
     vc = v_cache.transpose(1, 2).reshape(-1, kv_heads, dv).to(F64)

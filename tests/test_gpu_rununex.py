@@ -235,6 +235,41 @@ def test_prepare_and_masked_attention(case_, dtype):
             close(got, want, torch.float32 if what == "tails" else dtype, what, 3.0 if "attention" in what else 1.0)
 
 
+@pytest.mark.parametrize("heads,kv,maps,d,dv,chunk", [(8, 2, 2, 64, 128, 0), (20, 1, 1, 128, 64, 700), (4, 4, 1, 32, 32, 0)])
+def test_lone_tokens_with_their_keys_over_several_workgroups(heads, kv, maps, d, dv, chunk):
+    """A step of lone tokens after histories of unequal length: every token's key blocks shared out over 1, 3 and 8
+    workgroups and joined, against the plain version."""
+    g = torch.Generator().manual_seed(heads)
+    page = 16
+    step = PagedStep([300, 70, 5, 1029, 0], [1, 1, 1, 1, 1], page, seed=3)
+    T = 5
+    nk, nv = kv * maps * d, kv * dv
+    k_cache = torch.zeros(step.pages, page, nk, dtype=torch.bfloat16)
+    v_cache = torch.zeros(step.pages, nv, page, dtype=torch.bfloat16)
+    every = torch.tensor(step.old_rows() + step.rows.tolist())
+    k_cache.view(-1, nk)[every] = torch.randn(len(every), nk, generator=g).to(torch.bfloat16)
+    v_cache[every // page, :, every % page] = torch.randn(len(every), nv, generator=g).to(torch.bfloat16)
+    q = torch.randn(T, heads * maps * d, generator=g).to(torch.bfloat16)
+    sinks, r1, r2 = torch.randn(heads, generator=g), torch.rand(heads, generator=g), torch.rand(heads, generator=g) + 0.1
+    gate = torch.randn(T, heads * dv + 3, generator=g)
+    args = dict(chunk=chunk, r1=r1, r2=r2, sink=sinks, subtract=0.4, unit_eps=1e-5 if maps == 2 else None, out_scale=0.8,
+                gate=gate, gate_column=3)
+    want = reference_ops.masked_attention(q, k_cache, v_cache, step.tok_req, step.positions, step.table, page, heads, kv,
+                                          maps, d, dv, 0.17, **args)
+    plan = tiles_of(step)
+    assert not plan.info["any_portion"]
+    on_gpu = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in args.items()}
+    for splits in (1, 3, 8):
+        before = ops.masked_attention_force_splits(splits)
+        try:
+            got = ops.masked_attention(q.to(DEV), k_cache.to(DEV), v_cache.to(DEV), step.tok_req.to(DEV),
+                                       step.positions.to(DEV), step.table.to(DEV), page, heads, kv, maps, d, dv, 0.17,
+                                       plan=plan, max_ctx=1030 if splits > 1 else 0, **on_gpu)
+        finally:
+            ops.masked_attention_force_splits(before)
+        close(got.cpu(), want, torch.bfloat16, f"{splits} workgroups a token", 3.0)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("chunk,window,page", [(40, 0, 16), (7, 0, 4), (0, 25, 8), (300, 0, 16)])
 def test_one_key_carries_the_weight(dtype, chunk, window, page):
