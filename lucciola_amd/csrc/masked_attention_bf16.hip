@@ -50,6 +50,7 @@ struct MaskedArgs {
     bf16* out;
     float* shares;      // where a lone token's keys are shared out over workgroups: their sums, joined by a second kernel
     int zsplits;
+    int lone_only;      // the tiles of several tokens are another kernel's
 };
 
 // floats a wave leaves per lane and map where key ranges are joined: maximum, sum, the lane's part of O^T
@@ -73,15 +74,61 @@ struct ColumnState {
     floatx4 o[MAPS][DVB];       // O^T: value entries 16 t + 4 (lane / 16) + i of the lane's query column
 };
 
-// The lane's column: token row `tok`, head `head`, position `pos` (-1: no such column), first visible key `lo`.
-// Blocks first, first + stride, ... <= last of 16 keys each.
+// One block of 16 keys for the lane's column: scores from the keys' and the queries' operands, mask, bias, the running
+// maximum and sum, and the weighted values taken into O^T.
 template <int DSTEPS, int DVB, int MAPS>
-__device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const MaskedArgs& a, int g, int tok, int head,
-                                              int pos, int lo, const int* __restrict__ table, int first, int last,
-                                              int stride, int lane) {
-    const int quad = lane >> 4, col = lane & 15;
-    const size_t k_row = (size_t)a.kv_heads * MAPS * a.d;
-    bf16x8 bq[MAPS][DSTEPS];
+__device__ __forceinline__ void block_step(ColumnState<DVB, MAPS>& st, const MaskedArgs& a,
+                                           const bf16x8 (&bq)[MAPS][DSTEPS], const bf16x8 (&ka)[MAPS][DSTEPS],
+                                           const short4v (&va)[DVB], int key0, int pos, int lo, float bias1, float bias2,
+                                           int lane) {
+    const int quad = lane >> 4;
+    const int j0 = key0 + quad * 4;
+    float far[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) far[v] = a.r1 ? bias1 * __logf(1.f + bias2 * (float)max(pos - (j0 + v), 0)) : 0.f;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+        floatx4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < DSTEPS; ++i) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[m][i], bq[m][i], s, 0, 0, 0);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int j = j0 + v;
+            s[v] = (j >= lo && j <= pos) ? fmaf(s[v], a.scale, -far[v]) : -INFINITY;
+            mx = fmaxf(mx, s[v]);
+        }
+        mx = column_max4(mx);
+        const float m_new = fmaxf(st.m[m], mx);
+        const float base = m_new == -INFINITY ? 0.f : m_new;      // a column that has seen no key yet
+        const float alpha = __expf(st.m[m] - base);
+        float p[4], psum = 0.f;
+        short4v hi, lw;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            p[v] = __expf(s[v] - base);
+            psum += p[v];
+            const __bf16 top = (__bf16)p[v];
+            hi[v] = bits_of(top);
+            lw[v] = bits_of((__bf16)(p[v] - (float)top));
+        }
+        st.l[m] = fmaf(st.l[m], alpha, column_sum4(psum));
+        st.m[m] = m_new;
+        if (__any(alpha != 1.f))          // mostly the maximum stays where it is, and the rows as they are
+#pragma unroll
+            for (int t = 0; t < DVB; ++t) st.o[m][t] *= alpha;
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) {
+            st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], hi, st.o[m][t], 0, 0, 0);
+            st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], lw, st.o[m][t], 0, 0, 0);
+        }
+    }
+}
+
+template <int DSTEPS, int MAPS>
+__device__ __forceinline__ void load_queries(bf16x8 (&bq)[MAPS][DSTEPS], const MaskedArgs& a, int tok, int head, int pos,
+                                             int lane) {
+    const int quad = lane >> 4;
 #pragma unroll
     for (int m = 0; m < MAPS; ++m)
 #pragma unroll
@@ -92,7 +139,10 @@ __device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const 
             if (pos >= 0 && e < a.d)
                 bq[m][s] = *reinterpret_cast<const bf16x8*>(a.q + ((size_t)tok * a.heads + head) * MAPS * a.d + m * a.d + e);
         }
-    const float bias1 = (a.r1 && pos >= 0) ? a.r1[head] : 0.f, bias2 = (a.r1 && pos >= 0) ? a.r2[head] : 0.f;
+}
+
+template <int DVB, int MAPS>
+__device__ __forceinline__ void clear_state(ColumnState<DVB, MAPS>& st) {
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
         st.m[m] = -INFINITY;
@@ -100,6 +150,20 @@ __device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const 
 #pragma unroll
         for (int t = 0; t < DVB; ++t) st.o[m][t] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
+}
+
+// The lane's column: token row `tok`, head `head`, position `pos` (-1: no such column), first visible key `lo`.
+// Blocks first, first + stride, ... <= last of 16 keys each.
+template <int DSTEPS, int DVB, int MAPS>
+__device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const MaskedArgs& a, int g, int tok, int head,
+                                              int pos, int lo, const int* __restrict__ table, int first, int last,
+                                              int stride, int lane) {
+    const int quad = lane >> 4, col = lane & 15;
+    const size_t k_row = (size_t)a.kv_heads * MAPS * a.d;
+    bf16x8 bq[MAPS][DSTEPS];
+    load_queries<DSTEPS, MAPS>(bq, a, tok, head, pos, lane);
+    const float bias1 = (a.r1 && pos >= 0) ? a.r1[head] : 0.f, bias2 = (a.r1 && pos >= 0) ? a.r2[head] : 0.f;
+    clear_state<DVB, MAPS>(st);
     auto load_keys = [&](bf16x8 (&dst)[MAPS][DSTEPS], int b) {
         const int key0 = b * 16;
         const size_t row0 = (size_t)table[key0 / a.page_size] * a.page_size + key0 % a.page_size;
@@ -140,45 +204,7 @@ __device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const 
             load_keys(kn, b + stride);
             if constexpr (VALUES_AHEAD) load_values(vn, b + stride);
         }
-        const int j0 = key0 + quad * 4;
-        float far[4];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) far[v] = a.r1 ? bias1 * __logf(1.f + bias2 * (float)max(pos - (j0 + v), 0)) : 0.f;
-#pragma unroll
-        for (int m = 0; m < MAPS; ++m) {
-            floatx4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int i = 0; i < DSTEPS; ++i) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[m][i], bq[m][i], s, 0, 0, 0);
-            float mx = -INFINITY;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int j = j0 + v;
-                s[v] = (j >= lo && j <= pos) ? fmaf(s[v], a.scale, -far[v]) : -INFINITY;
-                mx = fmaxf(mx, s[v]);
-            }
-            mx = column_max4(mx);
-            const float m_new = fmaxf(st.m[m], mx);
-            const float base = m_new == -INFINITY ? 0.f : m_new;      // a column that has seen no key yet
-            const float alpha = __expf(st.m[m] - base);
-            float p[4], psum = 0.f;
-            short4v hi, lw;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                p[v] = __expf(s[v] - base);
-                psum += p[v];
-                const __bf16 top = (__bf16)p[v];
-                hi[v] = bits_of(top);
-                lw[v] = bits_of((__bf16)(p[v] - (float)top));
-            }
-            st.l[m] = fmaf(st.l[m], alpha, column_sum4(psum));
-            st.m[m] = m_new;
-#pragma unroll
-            for (int t = 0; t < DVB; ++t) {
-                st.o[m][t] *= alpha;
-                st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], hi, st.o[m][t], 0, 0, 0);
-                st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], lw, st.o[m][t], 0, 0, 0);
-            }
-        }
+        block_step<DSTEPS, DVB, MAPS>(st, a, bq, ka, va, key0, pos, lo, bias1, bias2, lane);
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
 #pragma unroll
@@ -254,7 +280,7 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
     };
     const bool lone = n == 1;
     const int z = blockIdx.z, zsplits = lone ? a.zsplits : 1;
-    if (!lone && z > 0) return;
+    if (!lone && (z > 0 || a.lone_only)) return;
     // head places of a pass (a power of two up to the waves), and the waves that share a place's keys
     int places = 1;
     if (!lone)
@@ -310,6 +336,7 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
         if (split == 0 && wave_on) {
             if (zsplits > 1) {
                 const int passes = (group + 15) / 16;
+                // [share][lane][map][numbers]: a lane's numbers in a row, which it reads back in wide loads
                 float* mine = a.shares + ((((size_t)blockIdx.x * a.kv_heads + g) * passes + h0 / 16) * zsplits + z)
                                              * kWave * MAPS * share_floats<DVB>() + (size_t)lane * MAPS * share_floats<DVB>();
 #pragma unroll
@@ -325,6 +352,160 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
                 finish_column<DVB, MAPS>(st, a, tok, head, pos, lane);
             }
         }
+    }
+}
+
+// Tiles of several tokens with their keys and values staged through LDS: all waves of the workgroup walk the same
+// stage (one block of 16 keys, or two where the waves of a head share out the blocks), which is fetched once for all of
+// them, the next stage travelling through registers while this one is worked on.  Keys lie in LDS as rows with 16 bytes
+// of padding, values transposed (a value entry's keys of the stage in a row, 16 bytes of padding): every operand is one
+// read without bank conflicts.  Lone tokens are left to the kernel above.
+constexpr int MB_STAGE_BLOCKS = 2;
+
+template <int DSTEPS, int DVB, int MAPS>
+__global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_staged_kernel(MaskedArgs a) {
+    extern __shared__ __align__(16) unsigned char staged[];       // two stages; afterwards where split key ranges meet
+    float (*meet)[kWave][DVB * 4 + 2] = reinterpret_cast<float (*)[kWave][DVB * 4 + 2]>(staged);
+    const int* tile = a.tiles + 4 * blockIdx.x;
+    const int t0 = tile[0], n = tile[1], r = tile[2], p0 = tile[3];
+    if (n == 1) return;
+    const int g = blockIdx.y, group = a.heads / a.kv_heads;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1), col = lane & 15, quad = lane >> 4;
+    const int* table = a.block_table + (size_t)r * a.max_blocks;
+    auto first_key = [&](int p) {
+        int lo = 0;
+        if (a.chunk > 0) lo = p - p % a.chunk;
+        if (a.window > 0) lo = max(lo, p - a.window + 1);
+        return lo;
+    };
+    int places = 1;
+    while (places < group && places < MB_WAVES) places *= 2;
+    const int splits = min(MB_WAVES / places, MB_STAGE_BLOCKS);      // blocks of a stage
+    const int place = wave % places, split = wave / places;
+    const int first = first_key(p0) / 16, last = (p0 + n - 1) / 16;
+    const int stages = (last - first + splits) / splits;
+    const int d_all = MAPS * a.d;                               // a key row's entries of this kv head
+    const int k_pitch = d_all * 2 + 16, v_pitch = splits * 32 + 16;                 // bytes
+    const int k_bytes = splits * 16 * k_pitch, stage_bytes = k_bytes + a.dv * v_pitch;
+    const size_t k_row = (size_t)a.kv_heads * d_all;
+    // what a thread fetches of a stage: 16-byte pieces of key rows, then of the transposed value rows
+    const int k_pieces = splits * 16 * (d_all / 8), v_pieces = splits * a.dv * 2;
+    constexpr int PIECES = 2;                                   // a thread's pieces of each kind at most
+    typedef int int4v __attribute__((ext_vector_type(4)));
+    int4v kreg[PIECES], vreg[PIECES];
+    auto fetch = [&](int stage) {
+        const int b0 = first + stage * splits;
+#pragma unroll
+        for (int u = 0; u < PIECES; ++u) {
+            const int i = threadIdx.x + u * MB_THREADS;
+            if (i < k_pieces) {
+                const int key = i / (d_all / 8), piece = i % (d_all / 8), b = b0 + key / 16;
+                if (b <= last) {
+                    const int key0 = b * 16;
+                    const size_t row = (size_t)table[key0 / a.page_size] * a.page_size + key0 % a.page_size + key % 16;
+                    kreg[u] = *reinterpret_cast<const int4v*>(a.k_cache + row * k_row + (size_t)g * d_all + piece * 8);
+                }
+            }
+            if (i < v_pieces) {
+                const int blk = i / (a.dv * 2), row = (i / 2) % a.dv, half = i & 1, b = b0 + blk;
+                if (b <= last) {
+                    const int key0 = b * 16;
+                    vreg[u] = *reinterpret_cast<const int4v*>(
+                        a.v_cache + ((size_t)table[key0 / a.page_size] * a.kv_heads * a.dv + (size_t)g * a.dv + row) * a.page_size
+                        + key0 % a.page_size + half * 8);
+                }
+            }
+        }
+    };
+    auto store = [&](int stage) {
+        unsigned char* base = staged + (size_t)(stage & 1) * stage_bytes;
+#pragma unroll
+        for (int u = 0; u < PIECES; ++u) {
+            const int i = threadIdx.x + u * MB_THREADS;
+            if (i < k_pieces) {
+                const int key = i / (d_all / 8), piece = i % (d_all / 8);
+                *reinterpret_cast<int4v*>(base + key * k_pitch + piece * 16) = kreg[u];
+            }
+            if (i < v_pieces) {
+                const int blk = i / (a.dv * 2), row = (i / 2) % a.dv, half = i & 1;
+                *reinterpret_cast<int4v*>(base + k_bytes + row * v_pitch + blk * 32 + half * 16) = vreg[u];
+            }
+        }
+    };
+    ColumnState<DVB, MAPS> st;
+    for (int h0 = 0; h0 < group; h0 += places) {
+        const int hh = h0 + place;
+        const bool wave_on = hh < group && split < splits;
+        const bool on = wave_on && col < n;
+        const int head = g * group + (hh < group ? hh : 0);
+        const int tok = t0 + (col < n ? col : 0);
+        const int pos = on ? p0 + col : -1;
+        const int lo = on ? first_key(pos) : 0;
+        bf16x8 bq[MAPS][DSTEPS];
+        load_queries<DSTEPS, MAPS>(bq, a, tok, head, pos, lane);
+        const float bias1 = (a.r1 && pos >= 0) ? a.r1[head] : 0.f, bias2 = (a.r1 && pos >= 0) ? a.r2[head] : 0.f;
+        clear_state<DVB, MAPS>(st);
+        __syncthreads();                    // the pass before this one has read its last stage
+        fetch(0);
+        store(0);
+        __syncthreads();
+        for (int stage = 0; stage < stages; ++stage) {
+            if (stage + 1 < stages) fetch(stage + 1);       // on its way while this stage is worked on
+            const int b = first + stage * splits + split;
+            if (wave_on && b <= last) {
+                const unsigned char* base = staged + (size_t)(stage & 1) * stage_bytes;
+                bf16x8 ka[MAPS][DSTEPS];
+                short4v va[DVB];
+#pragma unroll
+                for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+                    for (int i = 0; i < DSTEPS; ++i) {
+                        const int e = i * 32 + quad * 8;
+#pragma unroll
+                        for (int x = 0; x < 8; ++x) ka[m][i][x] = (__bf16)0.f;
+                        if (e < a.d)
+                            ka[m][i] = *reinterpret_cast<const bf16x8*>(base + (split * 16 + col) * k_pitch + (m * a.d + e) * 2);
+                    }
+#pragma unroll
+                for (int t = 0; t < DVB; ++t) {
+                    va[t] = short4v{0, 0, 0, 0};
+                    if (t * 16 < a.dv)
+                        va[t] = *reinterpret_cast<const short4v*>(base + k_bytes + (t * 16 + col) * v_pitch + split * 32 + quad * 8);
+                }
+                block_step<DSTEPS, DVB, MAPS>(st, a, bq, ka, va, b * 16, pos, lo, bias1, bias2, lane);
+            }
+            if (stage + 1 < stages) store(stage + 1);
+            __syncthreads();
+        }
+        if (splits > 1) {
+#pragma unroll
+            for (int m = 0; m < MAPS; ++m) {
+                __syncthreads();
+                if (split == 1 && wave_on) {
+                    float* mine = meet[place][lane];
+                    mine[0] = st.m[m];
+                    mine[1] = st.l[m];
+#pragma unroll
+                    for (int t = 0; t < DVB; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) mine[2 + t * 4 + i] = st.o[m][t][i];
+                }
+                __syncthreads();
+                if (split == 0 && wave_on) {
+                    const float* its = meet[place][lane];
+                    const float m_new = fmaxf(st.m[m], its[0]);
+                    const float base = m_new == -INFINITY ? 0.f : m_new;
+                    const float mine_by = expf(st.m[m] - base), its_by = expf(its[0] - base);
+                    st.l[m] = fmaf(st.l[m], mine_by, its[1] * its_by);
+#pragma unroll
+                    for (int t = 0; t < DVB; ++t)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) st.o[m][t][i] = fmaf(st.o[m][t][i], mine_by, its[2 + t * 4 + i] * its_by);
+                    st.m[m] = m_new;
+                }
+            }
+        }
+        if (split == 0 && wave_on) finish_column<DVB, MAPS>(st, a, tok, head, pos, lane);
     }
 }
 
@@ -372,6 +553,16 @@ __global__ __launch_bounds__(kWave) void masked_attention_bf16_join_kernel(Maske
 
 using namespace lc;
 
+static thread_local int g_staged = 1;
+
+// Tests and tuning: whether tiles of several tokens may take the kernel that stages keys and values in LDS (for the
+// calling thread).  Returns the setting before.
+LC_API int lc_masked_attention_bf16_staged(int on) {
+    const int before = g_staged;
+    if (on >= 0) g_staged = on ? 1 : 0;
+    return before;
+}
+
 // Whether the matrix-core kernel takes these sizes (else the general kernel serves them).
 LC_API int lc_masked_attention_bf16_supported(int d, int dv, int page_size, int maps) {
     return d > 0 && d % 8 == 0 && d <= 128 && dv > 0 && dv % 16 == 0 && dv <= 128 && page_size > 0 && page_size % 16 == 0
@@ -393,7 +584,8 @@ LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const vo
                                     int kv_heads, int maps, int d, int dv, float scale, int chunk, int window,
                                     const float* r1, const float* r2, const float* sink, float lambda, int unit_out,
                                     float eps, float out_scale, const float* gate, int gate_stride, int gate_column,
-                                    void* out, float* shares, int zsplits, hipStream_t stream) {
+                                    void* out, float* shares, int zsplits, int any_portion, int any_lone,
+                                    hipStream_t stream) {
     LC_CHECK(zsplits >= 1 && zsplits <= 64 && (zsplits == 1 || shares), "masked attention: bad shares");
     LC_CHECK(num_tiles >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && max_blocks > 0,
              "masked attention: bad sizes");
@@ -405,18 +597,32 @@ LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const vo
     LC_CHECK(kv_heads <= 65535, "masked attention: too many kv heads");
     MaskedArgs a{(const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, tiles, block_table, max_blocks, page_size,
                  heads, kv_heads, d, dv, scale, chunk, window, r1, r2, sink, lambda, unit_out, eps, out_scale, gate,
-                 gate_stride, gate_column, (bf16*)out, shares, zsplits};
+                 gate_stride, gate_column, (bf16*)out, shares, zsplits, 0};
+    // tiles of several tokens go through the kernel that stages keys and values in LDS where a stage fits a thread's
+    // two pieces of each kind
+    const int group = heads / kv_heads;
+    int places = 1;
+    while (places < group && places < MB_WAVES) places *= 2;
+    const int stage_blocks = MB_WAVES / places < MB_STAGE_BLOCKS ? MB_WAVES / places : MB_STAGE_BLOCKS;
+    const bool staged = any_portion && g_staged && stage_blocks * 16 * (maps * d / 8) <= 2 * MB_THREADS
+                        && stage_blocks * dv * 2 <= 2 * MB_THREADS;
+    size_t staged_lds = 2 * ((size_t)stage_blocks * 16 * (maps * d * 2 + 16) + (size_t)dv * (stage_blocks * 32 + 16));
+    const size_t meet_lds = (size_t)(MB_WAVES / 2) * kWave * (8 * 4 + 2) * sizeof(float);    // the same memory, later
+    if (staged_lds < meet_lds) staged_lds = meet_lds;
+    a.lone_only = staged ? 1 : 0;
+    const bool main_kernel = !staged || any_lone;
     const dim3 grid(num_tiles, kv_heads, zsplits), join_grid(num_tiles, kv_heads);
     const int dsteps = (d + 31) / 32, dvb = dv / 16;
-#define LC_MB(DS, VB)                                                                                                   \
+#define LC_MB_AS(DS, VB, MP)                                                                                            \
     do {                                                                                                                \
-        if (maps == 1) {                                                                                                \
-            masked_attention_bf16_kernel<DS, VB, 1><<<grid, MB_THREADS, 0, stream>>>(a);                                \
-            if (zsplits > 1) masked_attention_bf16_join_kernel<VB, 1><<<join_grid, kWave, 0, stream>>>(a);              \
-        } else {                                                                                                        \
-            masked_attention_bf16_kernel<DS, VB, 2><<<grid, MB_THREADS, 0, stream>>>(a);                                \
-            if (zsplits > 1) masked_attention_bf16_join_kernel<VB, 2><<<join_grid, kWave, 0, stream>>>(a);              \
-        }                                                                                                               \
+        if (staged) masked_attention_bf16_staged_kernel<DS, VB, MP><<<join_grid, MB_THREADS, staged_lds, stream>>>(a);  \
+        if (main_kernel) masked_attention_bf16_kernel<DS, VB, MP><<<grid, MB_THREADS, 0, stream>>>(a);                  \
+        if (zsplits > 1) masked_attention_bf16_join_kernel<VB, MP><<<join_grid, kWave, 0, stream>>>(a);                 \
+    } while (0)
+#define LC_MB(DS, VB)                          \
+    do {                                       \
+        if (maps == 1) LC_MB_AS(DS, VB, 1);    \
+        else LC_MB_AS(DS, VB, 2);              \
     } while (0)
 #define LC_MB_DV(DS)                     \
     do {                                 \
@@ -428,6 +634,7 @@ LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const vo
     else LC_MB_DV(4);
 #undef LC_MB_DV
 #undef LC_MB
+#undef LC_MB_AS
     LC_LAUNCH_CHECK("masked_attention_bf16");
     return 0;
 }

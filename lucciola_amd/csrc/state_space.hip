@@ -15,18 +15,17 @@ namespace lc {
 __device__ __forceinline__ float ss_silu(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float ss_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-// A thread per output entry.  proj [T, cols]: x (heads dv) | B (groups N) | C (groups N) | z (heads dv) | dt (heads);
+// A thread per convolved entry.  proj [T, cols]: x (heads dv) | B (groups N) | C (groups N) | z (heads dv) | dt (heads);
 // the first C = heads dv + 2 groups N columns pass the convolution.  Entry (t, i): i < heads dv is a channel of x;
-// the others are (head, n) pairs, whose thread makes the head's step and decay and its group's B and C at n (the
-// heads of a group each make their own copy of those two: a few multiply-adds against a trip through memory).
-// coef [3, T, heads N]; x_out [T, heads dv]
+// the others are (group, n) pairs, whose thread makes B and C at n and writes them for every head of the group with
+// the head's own step and decay.  coef [3, T, heads N]; x_out [T, heads dv]
 __global__ void state_space_prepare_kernel(const float* __restrict__ proj, int cols, int T, int heads, int groups,
                                            int N, int dv, const float* __restrict__ taps, const float* __restrict__ bias,
                                            int K, const float* __restrict__ tails, const float* __restrict__ dt_bias,
                                            const float* __restrict__ a_log, const int* __restrict__ tok_req,
                                            const int* __restrict__ q_offsets, const int* __restrict__ slot_ids,
                                            float* __restrict__ coef, float* __restrict__ x_out) {
-    const int inner = heads * dv, C = inner + 2 * groups * N, per_token = inner + heads * N;
+    const int inner = heads * dv, C = inner + 2 * groups * N, per_token = inner + groups * N, per_group = heads / groups;
     const size_t total = (size_t)T * per_token, plane = (size_t)T * heads * N;
     for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
          idx += (size_t)gridDim.x * blockDim.x) {
@@ -38,15 +37,18 @@ __global__ void state_space_prepare_kernel(const float* __restrict__ proj, int c
             x_out[(size_t)t * inner + i] = ss_silu(short_conv(proj, cols, t, local, i, taps, K, tail, C) + bias[i]);
             continue;
         }
-        const int head = (i - inner) / N, n = (i - inner) % N, g = head / (heads / groups);
+        const int g = (i - inner) / N, n = (i - inner) % N;
         const int cb = inner + g * N + n, cc = inner + groups * N + g * N + n;
         const float b = ss_silu(short_conv(proj, cols, t, local, cb, taps, K, tail, C) + bias[cb]);
         const float c = ss_silu(short_conv(proj, cols, t, local, cc, taps, K, tail, C) + bias[cc]);
-        const float step = ss_softplus(proj[(size_t)t * cols + C + inner + head] + dt_bias[head]);
-        const size_t at = (size_t)t * heads * N + (i - inner);
-        coef[at] = expf(-expf(a_log[head]) * step);
-        coef[plane + at] = step * b;
-        coef[2 * plane + at] = c;
+        for (int k = 0; k < per_group; ++k) {
+            const int head = g * per_group + k;
+            const float step = ss_softplus(proj[(size_t)t * cols + C + inner + head] + dt_bias[head]);
+            const size_t at = ((size_t)t * heads + head) * N + n;
+            coef[at] = expf(-expf(a_log[head]) * step);
+            coef[plane + at] = step * b;
+            coef[2 * plane + at] = c;
+        }
     }
 }
 
@@ -99,7 +101,7 @@ LC_API int lc_state_space_prepare(const float* proj, int cols, int T, int heads,
     if (T == 0) return 0;
     LC_CHECK(proj && taps && bias && dt_bias && a_log && tok_req && q_offsets && slot_ids && coef && x_out && (K == 1 || tails),
              "state space prepare: null pointer");
-    const size_t total = (size_t)T * heads * (dv + N);
+    const size_t total = (size_t)T * (heads * dv + groups * N);
     const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
     state_space_prepare_kernel<<<blocks, 256, 0, stream>>>(proj, cols, T, heads, groups, N, dv, taps, bias, K, tails, dt_bias,
                                                            a_log, tok_req, q_offsets, slot_ids, coef, x_out);

@@ -106,7 +106,8 @@ _SIGNATURES = {
     "lc_masked_attention": "pppi" + "ppp" + "ii" + "i" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
     "lc_attention_prepare": "p" + "iiiiiii" + "pip" + "ppp" + "pip" + "if" + "ppp" + "i" + "pip",
     "lc_masked_attention_bf16_supported": "iiii",
-    "lc_masked_attention_bf16": "ppp" + "pi" + "pii" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "ppip",
+    "lc_masked_attention_bf16": "ppp" + "pi" + "pii" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "ppiiip",
+    "lc_masked_attention_bf16_staged": "i",
     "lc_masked_attention_bf16_workspace": "iiiiii",
     "lc_state_space_prepare": "piiiiii" + "ppi" + "ppp" + "ppp" + "pp" + "p",
     "lc_state_space_readout": "pppiipiipifipip",
@@ -1179,7 +1180,8 @@ def plan_latent_attention(layout):
     # is done takes the longest that is left (the order changes no tile's result)
     tiles.sort(key=lambda t: -(t[3] + t[1]))
     return ({"tiles": np.asarray(tiles, dtype=np.int32).reshape(-1, 4)},
-            {"any_portion": any(t[1] > 1 for t in tiles), "num_tiles": len(tiles)})
+            {"any_portion": any(t[1] > 1 for t in tiles), "any_lone": any(t[1] == 1 for t in tiles),
+             "num_tiles": len(tiles)})
 
 
 def latent_attention(qa: torch.Tensor, heads: int, rank: int, rot: int, tok_req: torch.Tensor,
@@ -1824,6 +1826,12 @@ def masked_attention_matrix_cores(on: bool) -> bool:
     return before
 
 
+def masked_attention_staged(on: bool) -> bool:
+    """Tests and tuning: whether tiles of several tokens may take the matrix-core kernel that stages keys and values
+    in LDS (for the calling thread).  Returns the setting before."""
+    return bool(library().lc_masked_attention_bf16_staged(1 if on else 0))
+
+
 def masked_attention_on_matrix_cores(dtype: torch.dtype, d: int, dv: int, page_size: int, maps: int) -> bool:
     """Whether the matrix-core kernel serves these sizes: bfloat16, key heads of a multiple of 8 up to 128 entries,
     value heads of a multiple of 16 up to 128, pages of a multiple of 16 tokens."""
@@ -1929,12 +1937,12 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     out = torch.empty((T, heads * dv), dtype=q.dtype, device=q.device)
     if T and plan is not None and _masked_fast.on and masked_attention_on_matrix_cores(q.dtype, d, dv, page_size, maps):
         tiles = plan.arrays["tiles"]
-        # a step of lone tokens that leaves most of the card idle: every token's key blocks over several workgroups,
-        # a workgroup keeping two blocks a wave at least
+        # a step of lone tokens that leaves most of the card idle: every token's key blocks over several workgroups (a
+        # workgroup a CU in all), a workgroup keeping two blocks a wave at least
         zsplits, shares = 1, None
         if not plan.info.get("any_portion", True) and max_ctx > 0:
             reach = min(int(chunk) or max_ctx, int(window) or max_ctx, max_ctx)
-            zsplits = max(1, min(_masked_splits.forced or 512 // max(1, tiles.shape[0] * kv_heads), 16, reach // 256))
+            zsplits = max(1, min(_masked_splits.forced or 256 // max(1, tiles.shape[0] * kv_heads), 16, reach // 256))
             if zsplits > 1:
                 words = library().lc_masked_attention_bf16_workspace(tiles.shape[0], heads, kv_heads, maps, dv, zsplits)
                 shares = torch.empty((words,), dtype=torch.float32, device=q.device)
@@ -1942,7 +1950,8 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
               _ptr(block_table), block_table.shape[1], int(page_size), heads, kv_heads, maps, d, dv, float(scale),
               int(chunk), int(window), _ptr(r1), _ptr(r2), _ptr(sink), float(subtract), 0 if unit_eps is None else 1,
               float(unit_eps or 0.0), float(out_scale), _ptr(gate), gate.shape[1] if gate is not None else 0,
-              int(gate_column), _ptr(out), _ptr(shares), zsplits, _stream())
+              int(gate_column), _ptr(out), _ptr(shares), zsplits, 1 if plan.info.get("any_portion", True) else 0,
+              1 if plan.info.get("any_lone", True) else 0, _stream())
     elif T:
         _call("lc_masked_attention", _ptr(q), _ptr(k_cache), _ptr(v_cache), _dt(q), _ptr(tok_req), _ptr(positions),
               _ptr(block_table), block_table.shape[1], int(page_size), T, heads, kv_heads, maps, d, dv, float(scale),

@@ -220,17 +220,24 @@ def test_prepare_and_masked_attention(case_, dtype):
                                  d, dv, 0.21, chunk=chunk, window=window, r1=on(r1), r2=on(r2), sink=on(sinks),
                                  subtract=0.45, unit_eps=1e-5 if maps == 2 else None, out_scale=0.7,
                                  gate=pj if gate else None, gate_column=C)
-        fast = None
+        fast = plain = None
         if o is ops and ops.masked_attention_on_matrix_cores(dtype, d, dv, page, maps):
-            fast = o.masked_attention(q, kc, vc, lists["tok_req"], on(step.positions), on(step.table), page, heads, kv,
-                                      maps, d, dv, 0.21, chunk=chunk, window=window, r1=on(r1), r2=on(r2), sink=on(sinks),
-                                      subtract=0.45, unit_eps=1e-5 if maps == 2 else None, out_scale=0.7,
-                                      gate=pj if gate else None, gate_column=C, plan=tiles_of(step))
-        outs.append([t.cpu() if t is not None else None for t in (q, kc, vc, tl, out, fast)])
+            for staged in (True, False):     # tiles of several tokens with their keys staged in LDS, and straight from memory
+                before = ops.masked_attention_staged(staged)
+                try:
+                    got = o.masked_attention(q, kc, vc, lists["tok_req"], on(step.positions), on(step.table), page, heads,
+                                             kv, maps, d, dv, 0.21, chunk=chunk, window=window, r1=on(r1), r2=on(r2),
+                                             sink=on(sinks), subtract=0.45, unit_eps=1e-5 if maps == 2 else None,
+                                             out_scale=0.7, gate=pj if gate else None, gate_column=C, plan=tiles_of(step))
+                finally:
+                    ops.masked_attention_staged(before)
+                fast, plain = (got, plain) if staged else (fast, got)
+        outs.append([t.cpu() if t is not None else None for t in (q, kc, vc, tl, out, fast, plain)])
     if dtype == torch.bfloat16 and case_ in ATTENTION_CASES[6:]:
         assert outs[1][5] is not None, "the matrix-core kernel should take these sizes"
-    for got, want, what in zip(outs[1], outs[0] + [outs[0][4]], ("q", "key rows", "value rows", "tails", "attention",
-                                                                  "attention on the matrix cores")):
+    for got, want, what in zip(outs[1], outs[0][:5] + [outs[0][4]] * 2,
+                               ("q", "key rows", "value rows", "tails", "attention", "attention on the matrix cores (staged)",
+                                "attention on the matrix cores")):
         if want is not None and got is not None:
             close(got, want, torch.float32 if what == "tails" else dtype, what, 3.0 if "attention" in what else 1.0)
 
