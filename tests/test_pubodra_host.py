@@ -161,7 +161,7 @@ def test_latent_attention_planner():
                         first_position=[299, 0, 7, 100], block_size=16, single=False)
     arrays, info = ops.plan_latent_attention(layout)
     tiles = arrays["tiles"].tolist()
-    assert info == {"any_portion": True, "num_tiles": 6}
+    assert info == {"any_portion": True, "any_lone": True, "num_tiles": 6}
     assert sorted(tiles) == sorted([[0, 1, 0, 299], [1, 16, 1, 0], [17, 16, 1, 16], [33, 8, 1, 32], [41, 1, 2, 7],
                                     [42, 16, 3, 100]])
     ends = [t[3] + t[1] for t in tiles]
