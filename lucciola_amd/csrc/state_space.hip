@@ -52,8 +52,8 @@ __global__ void state_space_prepare_kernel(const float* __restrict__ proj, int c
     }
 }
 
-// One workgroup per token.  o, x float32 [T, n]; z float32: columns z_column .. + n of gates [T, gate_cols];
-// skip float32 [heads] (D); weight float32 [n]; the row is normed in `parts` equal parts.
+// One workgroup per token and part of the row.  o, x float32 [T, n]; z float32: columns z_column .. + n of gates
+// [T, gate_cols]; skip float32 [heads] (D); weight float32 [n]; the row is normed in `parts` equal parts.
 template <typename T>
 __global__ void state_space_readout_kernel(const float* __restrict__ o, const float* __restrict__ x,
                                            const float* __restrict__ gates, int gate_cols, int z_column,
@@ -62,21 +62,16 @@ __global__ void state_space_readout_kernel(const float* __restrict__ o, const fl
     extern __shared__ float y[];
     __shared__ float scratch[16];
     const size_t t = blockIdx.x;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const float xv = x[t * n + i];
-        y[i] = fmaf(skip[i / dv], xv, o[t * n + i]) * ss_silu(gates[t * gate_cols + z_column + i]);
+    const int width = n / parts, first = blockIdx.y * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const int at = first + i;
+        const float v = fmaf(skip[at / dv], x[t * n + at], o[t * n + at]) * ss_silu(gates[t * gate_cols + z_column + at]);
+        y[i] = v;                       // a thread meets its own entries only
+        ss = fmaf(v, v, ss);
     }
-    __syncthreads();
-    const int width = n / parts;
-    for (int part = 0; part < parts; ++part) {
-        float ss = 0.f;
-        for (int i = threadIdx.x; i < width; i += blockDim.x) ss = fmaf(y[part * width + i], y[part * width + i], ss);
-        const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
-        for (int i = threadIdx.x; i < width; i += blockDim.x) {
-            const int at = part * width + i;
-            out[t * n + at] = from_f32<T>(y[at] * inv * weight[at]);
-        }
-    }
+    const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) out[t * n + first + i] = from_f32<T>(y[i] * inv * weight[first + i]);
 }
 
 // out = a_scale a + b_scale b, float32 arithmetic
@@ -117,15 +112,18 @@ LC_API int lc_state_space_readout(const float* o, const float* x, const float* g
              "state space readout: bad sizes");
     if (T == 0) return 0;
     LC_CHECK(o && x && gates && skip && weight && out, "state space readout: null pointer");
-    const size_t lds = (size_t)n * sizeof(float);
-    LC_CHECK(lds <= 48 * 1024, "state space readout: rows of %d entries are too long", n);
-    const int threads = n >= 1024 ? 256 : (n >= 256 ? 128 : 64);
+    const int width = n / parts;
+    const size_t lds = (size_t)width * sizeof(float);
+    LC_CHECK(lds <= 48 * 1024, "state space readout: parts of %d entries are too long", width);
+    LC_CHECK(parts <= 65535, "state space readout: too many parts (%d)", parts);
+    const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+    const dim3 grid(T, parts);
     if (dt == DT_F32)
-        state_space_readout_kernel<float><<<T, threads, lds, stream>>>(o, x, gates, gate_cols, z_column, skip, dv, weight,
-                                                                       parts, eps, n, (float*)out);
+        state_space_readout_kernel<float><<<grid, threads, lds, stream>>>(o, x, gates, gate_cols, z_column, skip, dv, weight,
+                                                                          parts, eps, n, (float*)out);
     else if (dt == DT_BF16)
-        state_space_readout_kernel<bf16><<<T, threads, lds, stream>>>(o, x, gates, gate_cols, z_column, skip, dv, weight,
-                                                                      parts, eps, n, (bf16*)out);
+        state_space_readout_kernel<bf16><<<grid, threads, lds, stream>>>(o, x, gates, gate_cols, z_column, skip, dv, weight,
+                                                                         parts, eps, n, (bf16*)out);
     else
         LC_CHECK(false, "state space readout: unknown dtype %d", dt);
     LC_LAUNCH_CHECK("state_space_readout");
