@@ -9,7 +9,7 @@
 
 namespace lc {
 
-constexpr int SHORT_CONV_MAX_TAPS = 8;
+constexpr int SHORT_CONV_MAX_TAPS = 16;
 
 // Channel c (column c of proj) of token t, the `local`-th token of its request in this step.
 // proj [T, cols]; taps [C, K]; tail [K - 1, C] of the request's slot.

@@ -1793,7 +1793,7 @@ def lightning_readout(o: torch.Tensor, gates: torch.Tensor, gate_column: int, we
 
 # ------------------------------------------------------------------------------ masked attention
 MASKED_ATTENTION_MAX = 256      # entries of a key head and of a value head at most
-SHORT_CONV_MAX_TAPS = 8
+SHORT_CONV_MAX_TAPS = 16
 
 
 class _MaskedSwitch(threading.local):

@@ -554,7 +554,7 @@ def gated_activation_weighted(gu, kind, routing):
 
 
 MASKED_ATTENTION_MAX = 256
-SHORT_CONV_MAX_TAPS = 8
+SHORT_CONV_MAX_TAPS = 16
 
 
 def _convolved(proj, C, taps, tail, tok_req, q_offsets, slot_ids, bias=None):
