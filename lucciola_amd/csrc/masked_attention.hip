@@ -214,6 +214,64 @@ __global__ __launch_bounds__(MA_THREADS) void attention_prepare_kernel(
         }
 }
 
+// The same for steps without the unit norm, where nothing is summed over a head: a thread per pair of neighbouring
+// entries of the whole row (head sizes and the row's stride even), the pair's inputs and taps in wide loads.  The sums
+// and the rotation are written as in the kernel above, so both give the same bits.
+template <typename T>
+__global__ void attention_prepare_pairs_kernel(
+    const float* __restrict__ proj, int cols, int T_, int nq, int nk, int nv, int d, int dv,
+    const float* __restrict__ taps, int K, const float* __restrict__ tails, const int* __restrict__ tok_req,
+    const int* __restrict__ q_offsets, const int* __restrict__ slot_ids, const float* __restrict__ table, int rot,
+    const int* __restrict__ positions, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int* __restrict__ rows, int page_size) {
+    const int C = (nq + nk) * d + nv * dv, pairs = C / 2, q_cols = nq * d, qk_cols = (nq + nk) * d;
+    const size_t total = (size_t)T_ * pairs;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const int t = (int)(idx / pairs), c = 2 * (int)(idx % pairs);
+        const bool is_v = c >= qk_cols;
+        const int at = is_v ? (c - qk_cols) % dv : c % d;          // the pair's place in its head
+        float a, b;
+        if (taps) {
+            const int r = tok_req[t];
+            const int local = t - q_offsets[r];
+            const float* tail = tails + (size_t)slot_ids[r] * (K - 1) * C;
+            a = b = 0.f;
+            for (int back = K - 1; back >= 0; --back) {         // oldest input first
+                const float2 in = *reinterpret_cast<const float2*>(
+                    back <= local ? proj + (size_t)(t - back) * cols + c : tail + (size_t)((K - 1) - (back - local)) * C + c);
+                a = fmaf(taps[(size_t)c * K + (K - 1 - back)], in.x, a);
+                b = fmaf(taps[(size_t)(c + 1) * K + (K - 1 - back)], in.y, b);
+            }
+        } else {
+            const float2 in = *reinterpret_cast<const float2*>(proj + (size_t)t * cols + c);
+            a = in.x;
+            b = in.y;
+        }
+        if (table && !is_v && at + 1 < rot) {
+            const float* angle = table + (size_t)positions[t] * rot;
+            const float cs = angle[at / 2], sn = angle[rot / 2 + at / 2];
+            const float a0 = a, b0 = b;
+            a = a0 * cs - b0 * sn;
+            b = fmaf(b0, cs, a0 * sn);
+        }
+        if (c < q_cols) {
+            q_out[(size_t)t * q_cols + c] = from_f32<T>(a);
+            q_out[(size_t)t * q_cols + c + 1] = from_f32<T>(b);
+        } else if (rows && rows[t] >= 0) {
+            if (is_v) {
+                T* dst = v_cache + ((size_t)(rows[t] / page_size) * nv * dv + (c - qk_cols)) * page_size + rows[t] % page_size;
+                dst[0] = from_f32<T>(a);
+                dst[page_size] = from_f32<T>(b);
+            } else {
+                T* dst = k_cache + (size_t)rows[t] * nk * d + (c - q_cols);
+                dst[0] = from_f32<T>(a);
+                dst[1] = from_f32<T>(b);
+            }
+        }
+    }
+}
+
 }  // namespace lc
 
 using namespace lc;
@@ -252,6 +310,16 @@ LC_API int lc_masked_attention(const void* q, const void* k_cache, const void* v
     return 0;
 }
 
+static thread_local int g_prepare_pairs = 1;
+
+// Tests: whether steps without the unit norm may take the kernel with a thread per pair of entries (for the calling
+// thread).  Returns the setting before.
+LC_API int lc_attention_prepare_pairs(int on) {
+    const int before = g_prepare_pairs;
+    if (on >= 0) g_prepare_pairs = on ? 1 : 0;
+    return before;
+}
+
 LC_API int lc_attention_prepare(const float* proj, int cols, int T, int nq, int nk, int nv, int d, int dv,
                                 const float* taps, int K, const float* tails, const int* tok_req,
                                 const int* q_offsets, const int* slot_ids, const float* table, int rot,
@@ -266,6 +334,22 @@ LC_API int lc_attention_prepare(const float* proj, int cols, int T, int nq, int 
              "attention prepare: a convolution needs 1 to %d taps, the tails and the request lists", SHORT_CONV_MAX_TAPS);
     LC_CHECK(!table || (rot > 0 && rot % 2 == 0 && rot <= d && positions), "attention prepare: bad rotation");
     LC_CHECK(!rows || (k_cache && v_cache && page_size > 0), "attention prepare: rows without a cache");
+    if (!unit && d % 2 == 0 && dv % 2 == 0 && cols % 2 == 0 && g_prepare_pairs) {
+        const size_t total = (size_t)T * (((nq + nk) * d + nv * dv) / 2);
+        const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+        if (dt == DT_F32)
+            attention_prepare_pairs_kernel<float><<<blocks, 256, 0, stream>>>(
+                proj, cols, T, nq, nk, nv, d, dv, taps, K, tails, tok_req, q_offsets, slot_ids, table, rot, positions,
+                (float*)q_out, (float*)k_cache, (float*)v_cache, rows, page_size > 0 ? page_size : 1);
+        else if (dt == DT_BF16)
+            attention_prepare_pairs_kernel<bf16><<<blocks, 256, 0, stream>>>(
+                proj, cols, T, nq, nk, nv, d, dv, taps, K, tails, tok_req, q_offsets, slot_ids, table, rot, positions,
+                (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, rows, page_size > 0 ? page_size : 1);
+        else
+            LC_CHECK(false, "attention prepare: unknown dtype %d", dt);
+        LC_LAUNCH_CHECK("attention_prepare");
+        return 0;
+    }
     const int units = nq + nk + nv, per = MA_THREADS / kWave;
     const dim3 grid(T, (units + per - 1) / per);
     if (dt == DT_F32)

@@ -105,6 +105,7 @@ _SIGNATURES = {
     "lc_gated_activation_weighted": "ppippiiip",
     "lc_masked_attention": "pppi" + "ppp" + "ii" + "i" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "pp",
     "lc_attention_prepare": "p" + "iiiiiii" + "pip" + "ppp" + "pip" + "if" + "ppp" + "i" + "pip",
+    "lc_attention_prepare_pairs": "i",
     "lc_masked_attention_bf16_supported": "iiii",
     "lc_masked_attention_bf16": "ppp" + "pi" + "pii" + "iiiii" + "f" + "ii" + "ppp" + "f" + "i" + "ff" + "pii" + "ppiiip",
     "lc_masked_attention_bf16_staged": "i",
@@ -1824,6 +1825,12 @@ def masked_attention_matrix_cores(on: bool) -> bool:
     before = _masked_fast.on
     _masked_fast.on = bool(on)
     return before
+
+
+def attention_prepare_pairs(on: bool) -> bool:
+    """Tests: whether :func:`attention_prepare` without the unit norm may take the kernel with a thread per pair of
+    entries (for the calling thread).  Returns the setting before."""
+    return bool(library().lc_attention_prepare_pairs(1 if on else 0))
 
 
 def masked_attention_staged(on: bool) -> bool:

@@ -211,9 +211,17 @@ def test_prepare_and_masked_attention(case_, dtype):
         kc, vc, tl = on(k_cache), on(v_cache), on(tail)
         lists = dict(tok_req=on(step.tok_req), q_offsets=on(step.q_offsets), slot_ids=on(step.slot_ids))
         pj = on(proj)
-        q = o.attention_prepare(pj, nq, nk, nv, d, dv, dtype, kc, vc, on(step.rows),
-                                taps=on(conv), tail=tl, table=on(table), rot=rot, positions=on(step.positions),
-                                unit_eps=1e-5 if unit else None, **lists)
+        prepare = dict(taps=on(conv), tail=tl, table=on(table), rot=rot, positions=on(step.positions),
+                       unit_eps=1e-5 if unit else None, **lists)
+        q = o.attention_prepare(pj, nq, nk, nv, d, dv, dtype, kc, vc, on(step.rows), **prepare)
+        if o is ops and not unit:       # a wave a head and a thread a pair of entries: the same bits
+            before = ops.attention_prepare_pairs(False)
+            try:
+                kc2, vc2 = on(k_cache), on(v_cache)
+                q2 = o.attention_prepare(pj, nq, nk, nv, d, dv, dtype, kc2, vc2, on(step.rows), **prepare)
+            finally:
+                ops.attention_prepare_pairs(before)
+            assert torch.equal(q, q2) and torch.equal(kc, kc2) and torch.equal(vc, vc2)
         if taps > 1:
             o.conv_tail_update(pj, tl, C, taps, lists["q_offsets"], lists["slot_ids"], len(step.new))
         out = o.masked_attention(q, kc, vc, lists["tok_req"], on(step.positions), on(step.table), page, heads, kv, maps,
