@@ -300,7 +300,7 @@ def test_one_key_carries_the_weight(dtype, chunk, window, page):
     k_cache = torch.zeros(step.pages, page, heads * d, dtype=dtype, device=DEV)
     v_cache = torch.zeros(step.pages, heads * dv, page, dtype=dtype, device=DEV)
     places = step.rows.long().to(DEV)
-    for marked in (0, 1, 39, 40, 41, 279, 280, 299, 300, 305, 329):
+    for marked in (0, 1, 15, 16, 17, 39, 40, 41, 279, 280, 287, 288, 299, 300, 305, 329):
         k = k_rows.clone()
         k[marked, :] = 1.0
         v = v_rows.clone()
@@ -333,6 +333,35 @@ def test_one_key_carries_the_weight(dtype, chunk, window, page):
                 assert abs(float(out[at, 0]) - want) < 1e-2, (f"key {marked}, query {p} ({'lone' if lone else 'prompt'}, "
                                                               f"{'matrix cores' if fast else 'general'}): "
                                                               f"{float(out[at, 0]):.3f}, expected {want}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("page", [4, 16])
+def test_a_sink_that_takes_the_weight_and_one_that_takes_none(dtype, page):
+    """Every value is 3, so without a sink every output is 3 whatever the scores are.  A sink far above the scores
+    leaves the keys no weight (the output goes to 0), one far below changes nothing, and a sink as large as the one
+    visible key's score halves the first token's output; the other head has the opposite sink."""
+    heads, d, dv, length = 2, 16, 16, 70
+    step = PagedStep([0], [length], page, seed=page)
+    k_cache = torch.zeros(step.pages, page, heads * d, dtype=dtype, device=DEV)
+    v_cache = torch.full((step.pages, heads * dv, page), 3.0, dtype=dtype, device=DEV)
+    q = torch.zeros(length, heads * d, dtype=dtype, device=DEV)          # every score is 0
+    common = (k_cache, v_cache, torch.zeros(length, dtype=torch.int32, device=DEV), step.positions.to(DEV),
+              step.table.to(DEV), page, heads, heads, 1, d, dv, 1.0)
+    plans = [None]
+    if ops.masked_attention_on_matrix_cores(dtype, d, dv, page, 1):
+        from lucciola_amd.engine.batch import Plan
+        tiles = [[t0, min(16, length - t0), 0, t0] for t0 in range(0, length, 16)]
+        plans.append(Plan({"tiles": torch.tensor(tiles, dtype=torch.int32, device=DEV)}, {}))
+    for plan in plans:
+        for sinks, want in (([40.0, -40.0], [0.0, 3.0]), ([-40.0, 40.0], [3.0, 0.0])):
+            out = ops.masked_attention(q, *common, chunk=32, sink=torch.tensor(sinks, device=DEV), plan=plan).float().cpu()
+            for h in range(heads):
+                assert float((out[:, h * dv:(h + 1) * dv] - want[h]).abs().max()) < 1e-3, (sinks, h, plan is not None)
+        out = ops.masked_attention(q, *common, chunk=32, sink=torch.zeros(heads, device=DEV), plan=plan).float().cpu()
+        for p in range(length):         # p - p % 32 + 1 keys of score 0 beside a sink of 0
+            keys = p % 32 + 1
+            assert abs(float(out[p, 0]) - 3.0 * keys / (keys + 1)) < 2e-2, (p, float(out[p, 0]))
 
 
 @pytest.mark.parametrize("heads,groups,N,dv,taps,parts", [(4, 2, 16, 8, 3, 2), (3, 3, 7, 5, 5, 3), (6, 2, 32, 32, 4, 2),
