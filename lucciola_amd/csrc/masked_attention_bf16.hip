@@ -51,6 +51,7 @@ struct MaskedArgs {
     float* shares;      // where a lone token's keys are shared out over workgroups: their sums, joined by a second kernel
     int zsplits;
     int lone_only;      // the tiles of several tokens are another kernel's
+    int wave_blocks;    // blocks of a stage for every wave that shares a head's keys, in the kernel that stages them
 };
 
 // floats a wave leaves per lane and map where key ranges are joined: maximum, sum, the lane's part of O^T
@@ -70,17 +71,17 @@ __device__ __forceinline__ float column_sum4(float v) {
 
 template <int DVB, int MAPS>
 struct ColumnState {
-    float m[MAPS], l[MAPS];
+    float m[MAPS], l[MAPS];     // the column's reference point (the same in its four lanes); the lane's own part of the sum
     floatx4 o[MAPS][DVB];       // O^T: value entries 16 t + 4 (lane / 16) + i of the lane's query column
 };
 
-// One block of 16 keys for the lane's column: scores from the keys' and the queries' operands, mask, bias, the running
-// maximum and sum, and the weighted values taken into O^T.
+// One block of 16 keys for the lane's column: scores from the keys' and the queries' operands, mask, bias, the
+// reference point and the sum, and the weighted values taken into O^T.
 template <int DSTEPS, int DVB, int MAPS>
 __device__ __forceinline__ void block_step(ColumnState<DVB, MAPS>& st, const MaskedArgs& a,
                                            const bf16x8 (&bq)[MAPS][DSTEPS], const bf16x8 (&ka)[MAPS][DSTEPS],
                                            const short4v (&va)[DVB], int key0, int pos, int lo, float bias1, float bias2,
-                                           int lane) {
+                                           bool all_seen, int lane) {
     const int quad = lane >> 4;
     const int j0 = key0 + quad * 4;
     float far[4];
@@ -92,36 +93,55 @@ __device__ __forceinline__ void block_step(ColumnState<DVB, MAPS>& st, const Mas
 #pragma unroll
         for (int i = 0; i < DSTEPS; ++i) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[m][i], bq[m][i], s, 0, 0, 0);
         float mx = -INFINITY;
+        if (all_seen) {             // every column of the wave sees the whole block: nothing to mask
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int j = j0 + v;
-            s[v] = (j >= lo && j <= pos) ? fmaf(s[v], a.scale, -far[v]) : -INFINITY;
-            mx = fmaxf(mx, s[v]);
-        }
-        mx = column_max4(mx);
-        const float m_new = fmaxf(st.m[m], mx);
-        const float base = m_new == -INFINITY ? 0.f : m_new;      // a column that has seen no key yet
-        const float alpha = __expf(st.m[m] - base);
-        float p[4], psum = 0.f;
-        short4v hi, lw;
+            for (int v = 0; v < 4; ++v) {
+                s[v] = fmaf(s[v], a.scale, -far[v]);
+                mx = fmaxf(mx, s[v]);
+            }
+        } else {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            p[v] = __expf(s[v] - base);
-            psum += p[v];
-            const __bf16 top = (__bf16)p[v];
-            hi[v] = bits_of(top);
-            lw[v] = bits_of((__bf16)(p[v] - (float)top));
+            for (int v = 0; v < 4; ++v) {
+                const int j = j0 + v;
+                s[v] = (j >= lo && j <= pos) ? fmaf(s[v], a.scale, -far[v]) : -INFINITY;
+                mx = fmaxf(mx, s[v]);
+            }
         }
-        st.l[m] = fmaf(st.l[m], alpha, column_sum4(psum));
-        st.m[m] = m_new;
-        if (__any(alpha != 1.f))          // mostly the maximum stays where it is, and the rows as they are
+        // The column's reference point st.m moves only when a score outgrows it by e^8 (or it has none yet): until
+        // then no lane asks its column's other three, the weights are exp(s - reference) <= e^8, and a lane keeps
+        // its own part of the column's sum, which is added up when the column is finished.
+        if (__any(mx > st.m[m] + 8.f)) {
+            const float top = column_max4(mx);
+            const float m_new = top > st.m[m] + 8.f ? top : st.m[m];
+            const float alpha = m_new == st.m[m] ? 1.f : __expf(st.m[m] - m_new);       // 0 from no reference at all
+            st.l[m] *= alpha;
 #pragma unroll
             for (int t = 0; t < DVB; ++t) st.o[m][t] *= alpha;
-#pragma unroll
-        for (int t = 0; t < DVB; ++t) {
-            st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], hi, st.o[m][t], 0, 0, 0);
-            st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], lw, st.o[m][t], 0, 0, 0);
+            st.m[m] = m_new;
         }
+        const float base = st.m[m] == -INFINITY ? 0.f : st.m[m];      // a column that has seen no key yet
+        // A weight p >= 0 as two bfloat16 numbers: its upper 16 bits, and the upper 16 bits of what they leave
+        // (p minus them is exact in float32): together p to 2^-15 of itself.
+        float psum = 0.f;
+        unsigned hi_bits[4], lw_bits[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float p = __expf(s[v] - base);
+            psum += p;
+            const unsigned whole = __float_as_uint(p), upper = whole & 0xffff0000u;
+            hi_bits[v] = whole >> 16;
+            lw_bits[v] = __float_as_uint(p - __uint_as_float(upper)) >> 16;
+        }
+        typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+        const short4v hi = __builtin_bit_cast(short4v, uint2v{hi_bits[0] | (hi_bits[1] << 16), hi_bits[2] | (hi_bits[3] << 16)});
+        const short4v lw = __builtin_bit_cast(short4v, uint2v{lw_bits[0] | (lw_bits[1] << 16), lw_bits[2] | (lw_bits[3] << 16)});
+        st.l[m] += psum;
+        // the weights' upper halves into every block of value entries first, then the remainders: no product waits
+        // for the one before it
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], hi, st.o[m][t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < DVB; ++t) st.o[m][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va[t], lw, st.o[m][t], 0, 0, 0);
     }
 }
 
@@ -153,11 +173,12 @@ __device__ __forceinline__ void clear_state(ColumnState<DVB, MAPS>& st) {
 }
 
 // The lane's column: token row `tok`, head `head`, position `pos` (-1: no such column), first visible key `lo`.
-// Blocks first, first + stride, ... <= last of 16 keys each.
+// Blocks first, first + stride, ... <= last of 16 keys each.  Keys seen_from .. seen_to are seen by every column of
+// the tile (a block inside them needs no mask).
 template <int DSTEPS, int DVB, int MAPS>
 __device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const MaskedArgs& a, int g, int tok, int head,
                                               int pos, int lo, const int* __restrict__ table, int first, int last,
-                                              int stride, int lane) {
+                                              int stride, int seen_from, int seen_to, int lane) {
     const int quad = lane >> 4, col = lane & 15;
     const size_t k_row = (size_t)a.kv_heads * MAPS * a.d;
     bf16x8 bq[MAPS][DSTEPS];
@@ -204,7 +225,8 @@ __device__ __forceinline__ void attend_blocks(ColumnState<DVB, MAPS>& st, const 
             load_keys(kn, b + stride);
             if constexpr (VALUES_AHEAD) load_values(vn, b + stride);
         }
-        block_step<DSTEPS, DVB, MAPS>(st, a, bq, ka, va, key0, pos, lo, bias1, bias2, lane);
+        block_step<DSTEPS, DVB, MAPS>(st, a, bq, ka, va, key0, pos, lo, bias1, bias2,
+                                      key0 >= seen_from && key0 + 15 <= seen_to, lane);
 #pragma unroll
         for (int m = 0; m < MAPS; ++m)
 #pragma unroll
@@ -229,7 +251,7 @@ __device__ __forceinline__ void finish_column(const ColumnState<DVB, MAPS>& st, 
             sunk = expf(a.sink[head] - top);
         }
         const float shrink = pos >= 0 ? expf(st.m[m] - top) : 0.f;
-        const float denom = fmaf(st.l[m], shrink, sunk);
+        const float denom = fmaf(column_sum4(st.l[m]), shrink, sunk);        // the four lanes' parts of the column's sum
         const float w = denom > 0.f ? shrink / denom : 0.f;
 #pragma unroll
         for (int t = 0; t < DVB; ++t) {
@@ -289,6 +311,9 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
     const int place = wave % places, split = wave / places;
     // the blocks from the first token's first key to the last token
     const int first = first_key(p0) / 16, last = (p0 + n - 1) / 16;
+    // what every token of the tile sees: from the last token's first key to the first token (a column without a token
+    // or head computes on zeros there and is never written)
+    const int seen_from = first_key(p0 + n - 1), seen_to = p0;
     const int heads_a_pass = lone ? 16 : places;
     ColumnState<DVB, MAPS> st;
     for (int h0 = 0; h0 < group; h0 += heads_a_pass) {
@@ -302,7 +327,7 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
         const bool wave_on = lone || h0 + place < group;
         if (wave_on)
             attend_blocks<DSTEPS, DVB, MAPS>(st, a, g, tok, head, pos, lo, table, first + z * splits + split, last,
-                                             splits * zsplits, lane);
+                                             splits * zsplits, seen_from, seen_to, lane);
         if (splits > 1) {
 #pragma unroll
             for (int m = 0; m < MAPS; ++m) {
@@ -356,15 +381,17 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_kernel(Maske
 }
 
 // Tiles of several tokens with their keys and values staged through LDS: all waves of the workgroup walk the same
-// stage (one block of 16 keys, or two where the waves of a head share out the blocks), which is fetched once for all of
-// them, the next stage travelling through registers while this one is worked on.  Keys lie in LDS as rows with 16 bytes
-// of padding, values transposed (a value entry's keys of the stage in a row, 16 bytes of padding): every operand is one
-// read without bank conflicts.  Lone tokens are left to the kernel above.
+// stage, which is fetched once for all of them, the next stage travelling through registers while this one is worked
+// on.  A stage is `wave_blocks` blocks of 16 keys for every wave that shares a head's keys (one wave a head, or two
+// where the group has four heads or fewer): two blocks a wave where a thread's share of a stage is two 16-byte pieces
+// of keys and two of values at most, so that a stage's work outlasts the next one's trip from memory; else one.  Keys
+// lie in LDS as rows with 16 bytes of padding, values transposed (a value entry's keys of the stage in a row, 16 bytes
+// of padding): every operand is one read without bank conflicts.  Lone tokens are left to the kernel above.
 constexpr int MB_STAGE_BLOCKS = 2;
 
 template <int DSTEPS, int DVB, int MAPS>
 __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_staged_kernel(MaskedArgs a) {
-    extern __shared__ __align__(16) unsigned char staged[];       // two stages; afterwards where split key ranges meet
+    extern __shared__ __align__(16) unsigned char staged[];       // a stage; afterwards where split key ranges meet
     float (*meet)[kWave][DVB * 4 + 2] = reinterpret_cast<float (*)[kWave][DVB * 4 + 2]>(staged);
     const int* tile = a.tiles + 4 * blockIdx.x;
     const int t0 = tile[0], n = tile[1], r = tile[2], p0 = tile[3];
@@ -380,55 +407,72 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_staged_kerne
     };
     int places = 1;
     while (places < group && places < MB_WAVES) places *= 2;
-    const int splits = min(MB_WAVES / places, MB_STAGE_BLOCKS);      // blocks of a stage
+    const int splits = min(MB_WAVES / places, MB_STAGE_BLOCKS);      // waves that share a head's keys
     const int place = wave % places, split = wave / places;
     const int first = first_key(p0) / 16, last = (p0 + n - 1) / 16;
-    const int stages = (last - first + splits) / splits;
+    const int stage_blocks = splits * a.wave_blocks;
+    const int stages = (last - first + stage_blocks) / stage_blocks;
+    const int seen_from = first_key(p0 + n - 1);        // every token of the tile sees the keys from here to p0
+    const bool full_sizes = a.d == DSTEPS * 32 && a.dv == DVB * 16;
     const int d_all = MAPS * a.d;                               // a key row's entries of this kv head
-    const int k_pitch = d_all * 2 + 16, v_pitch = splits * 32 + 16;                 // bytes
-    const int k_bytes = splits * 16 * k_pitch, stage_bytes = k_bytes + a.dv * v_pitch;
+    const int k_pitch = d_all * 2 + 16, v_pitch = stage_blocks * 32 + 16;           // bytes
+    const int k_bytes = stage_blocks * 16 * k_pitch;
     const size_t k_row = (size_t)a.kv_heads * d_all;
-    // what a thread fetches of a stage: 16-byte pieces of key rows, then of the transposed value rows
-    const int k_pieces = splits * 16 * (d_all / 8), v_pieces = splits * a.dv * 2;
     constexpr int PIECES = 2;                                   // a thread's pieces of each kind at most
     typedef int int4v __attribute__((ext_vector_type(4)));
     int4v kreg[PIECES], vreg[PIECES];
+    // A thread's places in a stage are counted in units that the build knows (KP pieces a key row, DVB * 32 pieces a
+    // block of values: no division by a size that only the launch knows); places beyond the real sizes stay empty.
+    constexpr int KP = DSTEPS * 4 * MAPS, VP = DVB * 32, MAX_BLOCKS = 2 * MB_STAGE_BLOCKS;
     auto fetch = [&](int stage) {
-        const int b0 = first + stage * splits;
+        const int b0 = first + stage * stage_blocks;
+        int page_of[MAX_BLOCKS], within_of[MAX_BLOCKS];         // the same for all threads
+#pragma unroll
+        for (int blk = 0; blk < MAX_BLOCKS; ++blk) {
+            const int key0 = (b0 + blk) * 16;
+            const bool there = blk < stage_blocks && b0 + blk <= last;
+            page_of[blk] = there ? table[key0 / a.page_size] : -1;
+            within_of[blk] = key0 % a.page_size;
+        }
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             const int i = threadIdx.x + u * MB_THREADS;
-            if (i < k_pieces) {
-                const int key = i / (d_all / 8), piece = i % (d_all / 8), b = b0 + key / 16;
-                if (b <= last) {
-                    const int key0 = b * 16;
-                    const size_t row = (size_t)table[key0 / a.page_size] * a.page_size + key0 % a.page_size + key % 16;
+            {
+                const int key = i / KP, piece = i % KP, blk = key >> 4;
+                int page = -1, within = 0;
+#pragma unroll
+                for (int x = 0; x < MAX_BLOCKS; ++x)
+                    if (blk == x) { page = page_of[x]; within = within_of[x]; }
+                if (page >= 0 && piece * 8 < d_all) {
+                    const size_t row = (size_t)page * a.page_size + within + (key & 15);
                     kreg[u] = *reinterpret_cast<const int4v*>(a.k_cache + row * k_row + (size_t)g * d_all + piece * 8);
                 }
             }
-            if (i < v_pieces) {
-                const int blk = i / (a.dv * 2), row = (i / 2) % a.dv, half = i & 1, b = b0 + blk;
-                if (b <= last) {
-                    const int key0 = b * 16;
+            {
+                const int blk = i / VP, rem = i % VP, row = rem >> 1, half = rem & 1;
+                int page = -1, within = 0;
+#pragma unroll
+                for (int x = 0; x < MAX_BLOCKS; ++x)
+                    if (blk == x) { page = page_of[x]; within = within_of[x]; }
+                if (page >= 0 && row < a.dv)
                     vreg[u] = *reinterpret_cast<const int4v*>(
-                        a.v_cache + ((size_t)table[key0 / a.page_size] * a.kv_heads * a.dv + (size_t)g * a.dv + row) * a.page_size
-                        + key0 % a.page_size + half * 8);
-                }
+                        a.v_cache + ((size_t)page * a.kv_heads * a.dv + (size_t)g * a.dv + row) * a.page_size + within + half * 8);
             }
         }
     };
-    auto store = [&](int stage) {
-        unsigned char* base = staged + (size_t)(stage & 1) * stage_bytes;
+    auto store = [&]() {
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             const int i = threadIdx.x + u * MB_THREADS;
-            if (i < k_pieces) {
-                const int key = i / (d_all / 8), piece = i % (d_all / 8);
-                *reinterpret_cast<int4v*>(base + key * k_pitch + piece * 16) = kreg[u];
+            {
+                const int key = i / KP, piece = i % KP;
+                if (key < stage_blocks * 16 && piece * 8 < d_all)
+                    *reinterpret_cast<int4v*>(staged + key * k_pitch + piece * 16) = kreg[u];
             }
-            if (i < v_pieces) {
-                const int blk = i / (a.dv * 2), row = (i / 2) % a.dv, half = i & 1;
-                *reinterpret_cast<int4v*>(base + k_bytes + row * v_pitch + blk * 32 + half * 16) = vreg[u];
+            {
+                const int blk = i / VP, rem = i % VP, row = rem >> 1, half = rem & 1;
+                if (blk < stage_blocks && row < a.dv)
+                    *reinterpret_cast<int4v*>(staged + k_bytes + row * v_pitch + blk * 32 + half * 16) = vreg[u];
             }
         }
     };
@@ -447,34 +491,46 @@ __global__ __launch_bounds__(MB_THREADS) void masked_attention_bf16_staged_kerne
         clear_state<DVB, MAPS>(st);
         __syncthreads();                    // the pass before this one has read its last stage
         fetch(0);
-        store(0);
+        store();
         __syncthreads();
         for (int stage = 0; stage < stages; ++stage) {
             if (stage + 1 < stages) fetch(stage + 1);       // on its way while this stage is worked on
-            const int b = first + stage * splits + split;
-            if (wave_on && b <= last) {
-                const unsigned char* base = staged + (size_t)(stage & 1) * stage_bytes;
+            for (int j = 0; j < a.wave_blocks; ++j) {
+                const int blk = j * splits + split, b = first + stage * stage_blocks + blk;
+                if (!wave_on || b > last) continue;
                 bf16x8 ka[MAPS][DSTEPS];
                 short4v va[DVB];
+                const unsigned char* krow = staged + (blk * 16 + col) * k_pitch + quad * 16;
+                const unsigned char* vrow = staged + k_bytes + col * v_pitch + blk * 32 + quad * 8;
+                if (full_sizes) {           // the sizes the kernel is built for: no operand has empty places
 #pragma unroll
-                for (int m = 0; m < MAPS; ++m)
+                    for (int m = 0; m < MAPS; ++m)
 #pragma unroll
-                    for (int i = 0; i < DSTEPS; ++i) {
-                        const int e = i * 32 + quad * 8;
+                        for (int i = 0; i < DSTEPS; ++i)
+                            ka[m][i] = *reinterpret_cast<const bf16x8*>(krow + (m * DSTEPS * 32 + i * 32) * 2);
 #pragma unroll
-                        for (int x = 0; x < 8; ++x) ka[m][i][x] = (__bf16)0.f;
-                        if (e < a.d)
-                            ka[m][i] = *reinterpret_cast<const bf16x8*>(base + (split * 16 + col) * k_pitch + (m * a.d + e) * 2);
+                    for (int t = 0; t < DVB; ++t) va[t] = *reinterpret_cast<const short4v*>(vrow + t * 16 * v_pitch);
+                } else {
+#pragma unroll
+                    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+                        for (int i = 0; i < DSTEPS; ++i) {
+                            const int e = i * 32 + quad * 8;
+#pragma unroll
+                            for (int x = 0; x < 8; ++x) ka[m][i][x] = (__bf16)0.f;
+                            if (e < a.d) ka[m][i] = *reinterpret_cast<const bf16x8*>(krow + (m * a.d + i * 32) * 2);
+                        }
+#pragma unroll
+                    for (int t = 0; t < DVB; ++t) {
+                        va[t] = short4v{0, 0, 0, 0};
+                        if (t * 16 < a.dv) va[t] = *reinterpret_cast<const short4v*>(vrow + t * 16 * v_pitch);
                     }
-#pragma unroll
-                for (int t = 0; t < DVB; ++t) {
-                    va[t] = short4v{0, 0, 0, 0};
-                    if (t * 16 < a.dv)
-                        va[t] = *reinterpret_cast<const short4v*>(base + k_bytes + (t * 16 + col) * v_pitch + split * 32 + quad * 8);
                 }
-                block_step<DSTEPS, DVB, MAPS>(st, a, bq, ka, va, b * 16, pos, lo, bias1, bias2, lane);
+                block_step<DSTEPS, DVB, MAPS>(st, a, bq, ka, va, b * 16, pos, lo, bias1, bias2,
+                                              b * 16 >= seen_from && b * 16 + 15 <= p0, lane);
             }
-            if (stage + 1 < stages) store(stage + 1);
+            __syncthreads();                    // every wave has read the stage
+            if (stage + 1 < stages) store();
             __syncthreads();
         }
         if (splits > 1) {
@@ -597,16 +653,21 @@ LC_API int lc_masked_attention_bf16(const void* q, const void* k_cache, const vo
     LC_CHECK(kv_heads <= 65535, "masked attention: too many kv heads");
     MaskedArgs a{(const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, tiles, block_table, max_blocks, page_size,
                  heads, kv_heads, d, dv, scale, chunk, window, r1, r2, sink, lambda, unit_out, eps, out_scale, gate,
-                 gate_stride, gate_column, (bf16*)out, shares, zsplits, 0};
+                 gate_stride, gate_column, (bf16*)out, shares, zsplits, 0, 1};
     // tiles of several tokens go through the kernel that stages keys and values in LDS where a stage fits a thread's
     // two pieces of each kind
     const int group = heads / kv_heads;
     int places = 1;
     while (places < group && places < MB_WAVES) places *= 2;
-    const int stage_blocks = MB_WAVES / places < MB_STAGE_BLOCKS ? MB_WAVES / places : MB_STAGE_BLOCKS;
-    const bool staged = any_portion && g_staged && stage_blocks * 16 * (maps * d / 8) <= 2 * MB_THREADS
-                        && stage_blocks * dv * 2 <= 2 * MB_THREADS;
-    size_t staged_lds = 2 * ((size_t)stage_blocks * 16 * (maps * d * 2 + 16) + (size_t)dv * (stage_blocks * 32 + 16));
+    const int sharing = MB_WAVES / places < MB_STAGE_BLOCKS ? MB_WAVES / places : MB_STAGE_BLOCKS;
+    const int dsteps_built = (d + 31) / 32 <= 2 ? 2 : 4, dvb_built = dv <= 32 ? 2 : (dv <= 64 ? 4 : 8);
+    auto fits = [&](int blocks) {       // a thread's two places of each kind at most, in the units the kernels are built for
+        return blocks * 16 * (dsteps_built * 4 * maps) <= 2 * MB_THREADS && blocks * dvb_built * 32 <= 2 * MB_THREADS;
+    };
+    const bool staged = any_portion && g_staged && fits(sharing);
+    a.wave_blocks = fits(2 * sharing) ? 2 : 1;
+    const int stage_blocks = sharing * a.wave_blocks;
+    size_t staged_lds = (size_t)stage_blocks * 16 * (maps * d * 2 + 16) + (size_t)dv * (stage_blocks * 32 + 16);
     const size_t meet_lds = (size_t)(MB_WAVES / 2) * kWave * (8 * 4 + 2) * sizeof(float);    // the same memory, later
     if (staged_lds < meet_lds) staged_lds = meet_lds;
     a.lone_only = staged ? 1 : 0;
