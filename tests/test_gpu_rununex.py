@@ -174,6 +174,11 @@ ATTENTION_CASES = [
     (16, 4, 1, 128, 128, 16, 64, 0, 0, 0, True, True, True, True),
     (20, 1, 1, 64, 64, 32, 0, 90, 0, 0, True, True, True, True),
     (2, 2, 1, 24, 16, 48, 33, 0, 0, 8, False, False, True, False),
+    # groups of 3, 2 and 8 heads a kv head; sizes between the ones the kernel is built for
+    (6, 2, 2, 40, 80, 16, 70, 0, 3, 16, False, False, False, False),
+    (4, 2, 1, 72, 48, 16, 0, 0, 0, 0, True, True, True, True),
+    (8, 1, 2, 32, 32, 32, 50, 0, 2, 32, False, False, False, False),
+    (8, 1, 1, 104, 112, 16, 0, 40, 0, 0, True, True, False, True),
 ]
 
 
